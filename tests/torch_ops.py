@@ -70,9 +70,146 @@ class TorchOps:
     def place_tokens(self, ids, dest, source, tokens, count):
         ids[dest[:count].long()] = tokens[source[:count].long()]
 
-    def embed(self, token_ids, table, scale=1.0):
+    def embed(self, token_ids, table, scale=1.0, copies=1):
         out = table[token_ids.long()].float()
-        return out * scale if scale != 1.0 else out
+        out = out * scale if scale != 1.0 else out
+        return out.repeat(1, copies) if copies != 1 else out
+
+    def stream_norm(self, residual, terms, scales, mix, out_weights, in_weights, weight, eps, streams, center, out_dtype, rows=None):
+        """``residual`` float32 [T, S * H].  With terms: ``x_t <- sum_s mix[s, t] x_s + out[t] * y`` where ``y = sum_i scales[i]
+        terms[i]`` (mix None: identity, out None: ones), in place unless ``rows`` is given.  Returns the norm of
+        ``u = sum_s in[s] x_s`` (in None: ones) times ``weight``, for all rows or for ``rows``."""
+        t = residual.shape[0]
+        h = residual.shape[1] // streams
+        select = slice(None) if rows is None else rows.long()
+        x = residual.view(t, streams, h)[select]
+        if len(terms):
+            y = sum(float(s) * term[select].float() for s, term in zip(scales, terms))
+            mixed = x if mix is None else torch.einsum("st,nsh->nth", mix.float(), x)
+            weights = torch.ones(streams, device=x.device) if out_weights is None else out_weights.float()
+            x = mixed + weights[None, :, None] * y[:, None, :]
+            if rows is None:
+                residual.view(t, streams, h).copy_(x)
+        u = x.sum(1) if in_weights is None else torch.einsum("s,nsh->nh", in_weights.float(), x)
+        if center:
+            u = u - u.mean(-1, keepdim=True)
+        var = (u * u).mean(-1, keepdim=True)
+        return (u / torch.sqrt(var + eps) * weight.float()).to(out_dtype)
+
+    def gated_act_mul(self, gate_up, activation):
+        inter = gate_up.shape[-1] // 2
+        gate, up = gate_up[:, :inter].float(), gate_up[:, inter:].float()
+        if activation == "gelu_tanh":
+            act = 0.5 * gate * (1.0 + torch.tanh(0.7978845608028654 * (gate + 0.044715 * gate * gate * gate)))
+        elif activation == "silu":
+            act = gate * torch.sigmoid(gate)
+        else:
+            raise ValueError(activation)
+        return (act * up).to(gate_up.dtype)
+
+    # -- short convolution, recurrences -------------------------------------------------------
+    def short_conv(self, x, channels, weight, tail, slots, cu_q, max_q_len, activation="none", update_state=True):
+        """``x`` [T, >= channels]: the first ``channels`` columns pass ``y_t = sum_j w[:, j] u_(t - taps + 1 + j)`` per sequence,
+        the inputs before a portion's start come from ``tail[slot]`` ([taps - 1, channels], oldest first), which is then
+        brought up to date.  Returns [T, channels] in x's dtype."""
+        taps = weight.shape[1]
+        out = torch.empty((x.shape[0], channels), dtype=x.dtype, device=x.device)
+        bounds = cu_q.tolist()
+        for b, slot in enumerate(slots.tolist()):
+            lo, hi = bounds[b], bounds[b + 1]
+            u = x[lo:hi, :channels].float()
+            if taps > 1:
+                before = tail[slot].float() if tail is not None else torch.zeros((taps - 1, channels), device=x.device)
+                u = torch.cat([before, u], 0)
+            y = sum(weight[:, j].float() * u[j:j + hi - lo] for j in range(taps))
+            if activation == "silu":
+                y = y * torch.sigmoid(y)
+            out[lo:hi] = y.to(x.dtype)
+            if taps > 1 and tail is not None and update_state:
+                tail[slot] = u[u.shape[0] - (taps - 1):].to(tail.dtype)
+        return out
+
+    def rotate_pad_write(self, qkv, num_heads, num_kv_heads, dim, vdim, cached_dim, positions, cos, sin, slot_mapping, k_cache, v_cache, block_size, write_kv=True):
+        """Rotates the first ``2 * cos.shape[1]`` channels of every q and k head (halves layout), writes k and v into the
+        pages at ``cached_dim`` channels a head (zeros in the padding) and returns q as [T, heads * cached_dim]."""
+        t = qkv.shape[0]
+        q_size, k_size = num_heads * dim, num_kv_heads * dim
+        q = qkv[:, :q_size].float().view(t, num_heads, dim)
+        k = qkv[:, q_size:q_size + k_size].float().view(t, num_kv_heads, dim)
+        v = qkv[:, q_size + k_size:].float().view(t, num_kv_heads, vdim)
+        if cos is not None:
+            half = cos.shape[1]
+            c, s_ = cos[positions.long()][:, None, :], sin[positions.long()][:, None, :]
+
+            def rotate(x):
+                a, b = x[..., :half], x[..., half:2 * half]
+                return torch.cat([a * c - b * s_, b * c + a * s_, x[..., 2 * half:]], -1)
+
+            q, k = rotate(q), rotate(k)
+        out = torch.zeros((t, num_heads, cached_dim), dtype=qkv.dtype, device=qkv.device)
+        out[:, :, :dim] = q.to(qkv.dtype)
+        if write_kv:
+            page, offset = (slot_mapping // block_size).long(), (slot_mapping % block_size).long()
+            k_pad = torch.zeros((t, num_kv_heads, cached_dim), dtype=k_cache.dtype, device=qkv.device)
+            k_pad[:, :, :dim] = k.to(k_cache.dtype)
+            v_pad = torch.zeros((t, num_kv_heads, cached_dim), dtype=v_cache.dtype, device=qkv.device)
+            v_pad[:, :, :vdim] = v.to(v_cache.dtype)
+            k_cache[page, :, offset, :] = k_pad
+            v_cache[page, :, :, offset] = v_pad
+        return out.view(t, num_heads * cached_dim)
+
+    def recurrence_prepare(self, qkv, q_at, k_at, kv_heads, dim, unit, q_scale, decay_source, decay_at, heads, decay_columns, rate, bias, sign,
+                           beta_source, beta_at):
+        """-> qk float32 [T, kv_heads, 2, dim] (q then k of a head), decay float32 [T, decay_columns] =
+        ``exp(-rate[h] * softplus(sign * (z + bias)))``, beta float32 [T, heads] = ``sigmoid(b)`` or None."""
+        t = qkv.shape[0]
+        q = qkv[:, q_at:q_at + kv_heads * dim].float().view(t, kv_heads, dim)
+        k = qkv[:, k_at:k_at + kv_heads * dim].float().view(t, kv_heads, dim)
+        if unit:
+            q = q / torch.sqrt((q * q).sum(-1, keepdim=True) + 1e-6)
+            k = k / torch.sqrt((k * k).sum(-1, keepdim=True) + 1e-6)
+        qk = torch.stack([q * q_scale, k], 2).contiguous()
+        z = decay_source[:, decay_at:decay_at + decay_columns].float()
+        if bias is not None:
+            z = z + bias.float()
+        per_head = decay_columns // heads
+        decay = torch.exp(-rate.float().repeat_interleave(per_head)[None, :] * torch.nn.functional.softplus(sign * z)).contiguous()
+        beta = None
+        if beta_source is not None:
+            beta = torch.sigmoid(beta_source[:, beta_at:beta_at + heads].float()).contiguous()
+        return qk, decay, beta
+
+    def linear_scan(self, qk, v_source, v_at, decay, beta, state, slots, cu_q, max_q_len, heads, kv_heads, dim, vdim, delta):
+        """Per sequence and head, token by token from ``state[slot, head]`` ([dim, vdim] float32), which is written back:
+        ``S <- g S`` (rows); ``u = beta (v - S^T k)`` (delta) or ``u = v``; ``o = S^T q + (k . q) u``; ``S <- S + k u^T``.
+        Returns float32 [T, heads * vdim]."""
+        t = qk.shape[0]
+        out = torch.empty((t, heads, vdim), dtype=torch.float32, device=qk.device)
+        v = v_source[:, v_at:v_at + heads * vdim].float().view(t, heads, vdim)
+        g = decay.view(t, heads, -1)
+        repeat = heads // kv_heads
+        bounds = cu_q.tolist()
+        for b, slot in enumerate(slots.tolist()):
+            s = state[slot].clone()  # [heads, dim, vdim]
+            for i in range(bounds[b], bounds[b + 1]):
+                q = qk[i, :, 0].repeat_interleave(repeat, 0)  # [heads, dim]
+                k = qk[i, :, 1].repeat_interleave(repeat, 0)
+                s = s * g[i][:, :, None]
+                u = v[i]
+                if delta:
+                    u = beta[i][:, None] * (u - torch.einsum("hde,hd->he", s, k))
+                out[i] = torch.einsum("hde,hd->he", s, q) + (k * q).sum(-1, keepdim=True) * u
+                s = s + k[:, :, None] * u[:, None, :]
+            state[slot] = s
+        return out.view(t, heads * vdim)
+
+    def gated_head_norm(self, read, weight, eps, gate_source, gate_at, gate_kind, heads, vdim, out_dtype):
+        t = read.shape[0]
+        o = read.view(t, heads, vdim)
+        o = o / torch.sqrt((o * o).mean(-1, keepdim=True) + eps) * weight.float()
+        gate = gate_source[:, gate_at:gate_at + heads * vdim].float().view(t, heads, vdim)
+        gate = gate * torch.sigmoid(gate) if gate_kind == "silu" else torch.sigmoid(gate)
+        return (o * gate).view(t, heads * vdim).to(out_dtype)
 
     @staticmethod
     def _one_delta(delta):

@@ -8,7 +8,9 @@ every entry in it (the reference has exactly one such group for all layers,
 as every key in them lies behind the window of all queries still to come.  Entries with
 a ``StateNeed`` get one row per request in fixed-size tensors, indexed by the request's
 *slot* (the reference's ``seq_index``, ``engine/scheduler.py:58,113-129``); slot rows are zeroed
-when a request takes the slot.
+when a request takes the slot.  An entry may state several needs at once (``CompositeNeed``: pages
+for keys beside a fixed-size state, or the needs of the mixers a mixer is made of); its leaves are
+treated like the needs of entries of their own and the mixer gets a ``CompositeView`` of the same form.
 
 What a page holds is the need's to say (``PagedNeed.tensors``: names, shapes per page and
 dtypes): per entry of a group every named tensor is ``[pages, *shape of one page]``, with the
@@ -27,7 +29,7 @@ from typing import Dict, List, Optional, Sequence, Tuple
 import numpy as np
 import torch
 
-from ..parts.base import PAGE, PagedNeed, StateNeed
+from ..parts.base import PAGE, CompositeNeed, PagedNeed, StateNeed
 from .allocator import NULL_PAGE, PoolExhausted, PageAllocator
 from .prefix import PrefixCache
 
@@ -153,6 +155,13 @@ class StateView:
     tensors: Dict[str, torch.Tensor]
 
 
+@dataclass
+class CompositeView:
+    """What a mixer with a ``CompositeNeed`` is handed: one view (or None) per part of the need, in its order."""
+
+    views: Tuple[object, ...]
+
+
 class CacheManager:
     def __init__(
         self,
@@ -173,16 +182,26 @@ class CacheManager:
         self.dtype = dtype
         self.device = torch.device(device)
         self.groups: List[PageGroup] = []
-        self.entry_group: Dict[int, Tuple[int, int]] = {}
+        self.entry_group: Dict[object, Tuple[int, int]] = {}
         by_need: Dict[PagedNeed, List[int]] = {}
         state_needs: Dict[int, StateNeed] = {}
-        for entry, need in enumerate(needs):
+        self.composite: Dict[object, CompositeNeed] = {}
+
+        def note(key, need) -> None:
+            # (a leaf of a composite need is keyed by (entry, place among the parts, ...) and is otherwise an entry like any other)
             if isinstance(need, PagedNeed):
-                by_need.setdefault(need, []).append(entry)
+                by_need.setdefault(need, []).append(key)
             elif isinstance(need, StateNeed):
-                state_needs[entry] = need
+                state_needs[key] = need
+            elif isinstance(need, CompositeNeed):
+                self.composite[key] = need
+                for place, part in enumerate(need.parts):
+                    note((key if isinstance(key, tuple) else (key,)) + (place,), part)
             elif need is not None:
-                raise TypeError(f"schedule entry {entry}: unknown cache need {need!r}")
+                raise TypeError(f"schedule entry {key}: unknown cache need {need!r}")
+
+        for entry, need in enumerate(needs):
+            note(entry, need)
         for need, entries in by_need.items():
             index = len(self.groups)
             self.groups.append(PageGroup(need, entries, num_pages, page_size, dtype, self.device, allocate_tensors, scatter_pages))
@@ -347,7 +366,10 @@ class CacheManager:
         return page * self.page_size + token_index % self.page_size
 
     # -- views handed to the mixers ----------------------------------------------------------
-    def view(self, entry: int, group_batches: Sequence[object]):
+    def view(self, entry, group_batches: Sequence[object]):
+        if entry in self.composite:
+            base = entry if isinstance(entry, tuple) else (entry,)
+            return CompositeView(tuple(self.view(base + (place,), group_batches) for place in range(len(self.composite[entry].parts))))
         if entry in self.entry_group:
             g, position = self.entry_group[entry]
             group = self.groups[g]

@@ -48,7 +48,8 @@ class Param:
     ``stored`` tensor stays in 32-bit when the checkpoint holds it so (a router's
     weights, say) and takes the run dtype otherwise.  ``product`` = False marks a
     matrix that no matrix product reads (a table that is only looked up).  ``init`` names the random-weights law: ``normal`` is
-    N(0, 0.02), ``one_plus_normal`` is 1 + N(0, 0.02).
+    N(0, 0.02), ``one_plus_normal`` is 1 + N(0, 0.02), ``identity_plus_normal`` the identity matrix + N(0, 0.02), ``mean_plus_normal``
+    1 / (first size) + N(0, 0.02).
     """
 
     shape: Tuple[int, ...]
@@ -176,6 +177,36 @@ class StateNeed:
     """Per-request state of fixed size: ``(name, shape, dtype)`` per tensor, dtype None = run dtype."""
 
     tensors: Tuple[Tuple[str, Tuple[int, ...], Optional[torch.dtype]], ...]
+
+
+@dataclass(frozen=True)
+class CompositeNeed:
+    """Several needs of one schedule entry: a mixer that keeps keys in pages AND a fixed-size state (the inputs a short
+    convolution still has to see, say), or a mixer that is made of mixers.  ``parts`` are ``PagedNeed``, ``StateNeed``,
+    ``CompositeNeed`` or None; the mixer is handed a ``CompositeView`` whose ``views`` stand in the same order."""
+
+    parts: Tuple[object, ...]
+
+
+@dataclass
+class ScaledSum:
+    """What a sub-layer made of two side by side hands on: ``scales[0] * terms[0] + scales[1] * terms[1]``, each term
+    ``[T, H]``; whoever adds it to the residual forms the sum in float32."""
+
+    terms: Tuple[torch.Tensor, ...]
+    scales: Tuple[float, ...]
+
+
+@dataclass
+class StreamUpdate:
+    """A sub-layer's output that the residual STREAMS have not taken in yet: ``x_t <- sum_s mix[s, t] x_s + out[t] * y``
+    for all streams at once.  ``y`` is ``[T, H]`` or a ``ScaledSum``; ``mix`` float32 ``[S, S]`` indexed [from, to],
+    ``out`` float32 ``[S]`` (None: the identity and ones, which is the plain residual sum).  The norm that reads the
+    streams next applies it inside its own kernel."""
+
+    y: object
+    mix: Optional[torch.Tensor] = None
+    out: Optional[torch.Tensor] = None
 
 
 @dataclass

@@ -11,6 +11,9 @@ on is the updated residual in the run dtype (``ResidualCopy``), which the norm's
 
 ``ParallelBlock`` (not in the reference): ``n = norm(h); h = h + (mixer(n) + ff(n))``, one norm that both
 sub-layers read.  It hands both outputs on as a ``SumOf``, which the next norm's kernel adds up in float32.
+
+``HyperConnectionBlock`` (not in the reference): pre-norm sub-layers over several copies of the residual that are read
+through learned weights and mixed by a learned matrix at every sub-layer.
 """
 from __future__ import annotations
 
@@ -18,7 +21,7 @@ from typing import Optional, Tuple
 
 import torch
 
-from .base import Block, FeedForward, Mixer, Norm, OutputNormSink, Part, ResidualCopy, ResidualSink, SumOf, register_arrangement
+from .base import Block, FeedForward, Mixer, Norm, OutputNormSink, Part, ResidualCopy, ResidualSink, StreamUpdate, SumOf, register_arrangement
 
 
 class PreNormBlock(Block):
@@ -133,3 +136,68 @@ class OutputNormBlock(Block):
 
 
 register_arrangement("output_norm", OutputNormBlock)
+
+
+class HyperConnectionBlock(Block):
+    """Pre-norm sub-layers over ``streams`` copies of the residual (hyper-connections): for sub-layer ``q`` with learned
+    ``in_q [S]``, ``out_q [S]`` and ``mix_q [S, S]`` (indexed [from, to]),
+
+        ``u = sum_s in_q[s] x_s``;  ``y = sublayer(norm_q(u))``;  ``x_t <- sum_s mix_q[s, t] x_s + out_q[t] y``  (all ``t`` at once).
+
+    The residual is float32 ``[T, S * H]``.  A sub-layer's output is not worked into the streams by a pass of its own:
+    it is handed on as a ``StreamUpdate`` and the next norm's kernel (``StreamNorm``) applies it before it reads the
+    streams, as the plain residual sum is folded into the next norm for the other arrangements.  The block's own tensors
+    are ``<prefix>hc1.{in,out,mix}`` and ``<prefix>hc2.{in,out,mix}`` (``names`` replaces the two prefixes)."""
+
+    def __init__(self, prefix: str, mixer: Mixer, feed_forward: FeedForward, mixer_norm: Norm, ff_norm: Norm, streams: int = 1,
+                 names: Tuple[str, str] = ("hc1.", "hc2."), learned: bool = True) -> None:
+        """``learned`` False: no tensors of the block's own; every stream is read with weight 1, keeps itself and takes
+        the output with weight 1 (with one stream: the plain pre-norm block, which may also go without a feed-forward)."""
+        super().__init__(prefix)
+        self.learned = bool(learned)
+        self.mixer = mixer
+        self.feed_forward = feed_forward
+        self.mixer_norm = mixer_norm
+        self.ff_norm = ff_norm
+        self.streams = int(streams)
+        self.names = tuple(names)
+        self.has_feed_forward = type(feed_forward).__name__ != "NoFeedForward"
+        for norm in (mixer_norm, ff_norm):
+            if getattr(norm, "streams", None) != self.streams or not hasattr(norm, "forward_streams"):
+                raise ValueError(f"a block over {self.streams} streams needs norms over as many (the 'stream_norm' kind)")
+        self.in1 = self.out1 = self.mix1 = self.in2 = self.out2 = self.mix2 = None
+
+    def children(self) -> Tuple[Part, ...]:
+        if not self.has_feed_forward:
+            return (self.mixer_norm, self.mixer)  # (no second norm: its tensor does not exist)
+        return (self.mixer_norm, self.mixer, self.ff_norm, self.feed_forward)
+
+    def params(self):
+        from .base import single
+
+        s = self.streams
+        out = {}
+        if not self.learned:
+            return out
+        for number, name in ((1, self.names[0]), (2, self.names[1])):
+            if number == 2 and not self.has_feed_forward:
+                break
+            out[f"in{number}"] = single(name + "in", (s,), role="vector", init="mean_plus_normal")
+            out[f"out{number}"] = single(name + "out", (s,), role="vector", init="one_plus_normal")
+            out[f"mix{number}"] = single(name + "mix", (s, s), role="vector", init="identity_plus_normal")
+        return out
+
+    def input_norm(self) -> Optional[Norm]:
+        return self.mixer_norm
+
+    def forward(self, residual: torch.Tensor, pending, ctx, cache, owns_cache: bool, next_norm: Optional[Norm] = None):
+        normed = self.mixer_norm.forward_streams(residual, pending, self.in1, ctx)
+        mixed = self.mixer.forward(normed, ctx, cache, owns_cache)
+        update = StreamUpdate(mixed, self.mix1, self.out1)
+        if not self.has_feed_forward:
+            return update
+        normed = self.ff_norm.forward_streams(residual, update, self.in2, ctx)
+        return StreamUpdate(self.feed_forward.forward(normed, ctx), self.mix2, self.out2)
+
+
+register_arrangement("hyper_connection", HyperConnectionBlock)

@@ -31,8 +31,9 @@ class GatedMLP(FeedForward):
         """``names``: the gate, up and down tensors below the prefix."""
         super().__init__(prefix)
         self.names = tuple(names)
-        if activation != "silu":
-            raise ValueError(f"activation {activation!r} is not implemented (only 'silu')")
+        if activation not in ("silu", "gelu_tanh"):
+            raise ValueError(f"activation {activation!r} is not implemented ('silu' or 'gelu_tanh')")
+        self.activation = activation
         self.hidden_size = int(hidden_size)
         self.intermediate_size = int(intermediate_size)
         self.gate_up_weight: Optional[torch.Tensor] = None
@@ -54,7 +55,11 @@ class GatedMLP(FeedForward):
 
     def forward(self, x, ctx, sink=None, partials_ok: bool = True):
         ops = ctx.ops
-        act = ops.linear_silu_mul(x, self.operand("gate_up_weight"), ctx.dtype)
+        if self.activation == "silu":
+            act = ops.linear_silu_mul(x, self.operand("gate_up_weight"), ctx.dtype)
+        else:
+            # gelu_tanh(z) = z / 2 * (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3))), in float32 with one rounding at the store
+            act = ops.gated_act_mul(ops.linear(x, self.operand("gate_up_weight"), None, ctx.dtype), self.activation)
         return ops.linear(act, self.operand("down_weight"), None, ctx.dtype, partials_ok=partials_ok, residual_norm=sink)
 
 

@@ -67,6 +67,9 @@ class ModelSpec:
     # head, ``tied_to`` (the table's checkpoint name or None).
     embedding: Optional[PartSpec] = None
     head: Optional[PartSpec] = None
+    # Copies of the residual that the blocks keep side by side (hyper-connections): the residual is then float32
+    # ``[T, residual_streams * H]``, every copy starts as the embedding output, and the final norm reads their sum.
+    residual_streams: int = 1
 
     def validate(self) -> None:
         if not self.layers:
@@ -96,7 +99,10 @@ class TableEmbedding(Embedding):
     def params(self) -> Dict[str, Param]:
         return {"table": single(self.name, (self.vocab_size, self.hidden_size), product=False)}
 
-    def forward(self, token_ids: torch.Tensor, ctx) -> torch.Tensor:
+    def forward(self, token_ids: torch.Tensor, ctx, copies: int = 1) -> torch.Tensor:
+        """``copies`` > 1: the row is written that many times side by side, ``[T, copies * H]``."""
+        if copies != 1:
+            return ctx.ops.embed(token_ids, self.table, scale=self.scale, copies=copies)
         if self.scale == 1.0:
             return ctx.ops.embed(token_ids, self.table)
         return ctx.ops.embed(token_ids, self.table, scale=self.scale)
@@ -187,10 +193,13 @@ class DecoderModel(Part):
     # -- arithmetic ---------------------------------------------------------------------
     def embed(self, token_ids: torch.Tensor, ctx) -> torch.Tensor:
         """The residual stream before the first block: float32 ``[T, H]``."""
+        streams = self.spec.residual_streams
+        if streams > 1 and self.spec.embedding_position is None:
+            return self.embedding.forward(token_ids, ctx, copies=streams)  # (the looked-up row written once per stream)
         residual = self.embedding.forward(token_ids, ctx)
         if self.spec.embedding_position is not None:
             residual = self.positions[self.spec.embedding_position].on_embeddings(residual, ctx)
-        return residual
+        return residual.repeat(1, streams) if streams > 1 else residual
 
     def run_schedule(self, residual: torch.Tensor, pending, ctx, first: int = 0, last: Optional[int] = None):
         """Runs schedule entries ``first .. last - 1`` on ``residual`` (updated in place); takes and returns ``pending``,

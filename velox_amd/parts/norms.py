@@ -1,4 +1,4 @@
-"""RMSNorm that owns the residual update.
+"""Norms that own the residual update: RMSNorm, and a norm over several residual streams (``StreamNorm``).
 
 Formula (reference ``src/rmsnorm.py:20-28``): in float32, ``y = x * rsqrt(mean(x^2) + eps) * w``,
 one rounding at the store.  The reference adds the residual in the model dtype
@@ -12,7 +12,7 @@ from typing import Dict, Optional
 
 import torch
 
-from .base import DeferredNorm, Norm, Param, ResidualCopy, register_part, single
+from .base import DeferredNorm, Norm, Param, ResidualCopy, ScaledSum, StreamUpdate, register_part, single
 
 
 class RMSNorm(Norm):
@@ -49,3 +49,52 @@ class RMSNorm(Norm):
 
 
 register_part("norm", "rmsnorm", RMSNorm)
+
+
+class StreamNorm(Norm):
+    """A norm with a weight and no bias over ``streams`` copies of the residual: the residual is float32 ``[T, streams * H]``
+    (one stream after the other within a token's row), the norm reads ``u = sum_s in[s] x_s`` (``in`` None: the plain sum)
+    and gives ``(u - mean(u)) / sqrt(var(u) + eps) * w`` (``center``, a layer norm without bias) or ``u / sqrt(mean(u^2) +
+    eps) * w``.  What the sub-layer before it produced reaches it as a ``StreamUpdate`` and is worked into the streams
+    by the same kernel, before they are read.  With one stream and no weights on the streams this is the plain
+    ``residual += delta; normalise(residual)``."""
+
+    def __init__(self, prefix: str, hidden_size: int, eps: float, weight_name: str = "weight", streams: int = 1, center: bool = True) -> None:
+        super().__init__(prefix)
+        if int(streams) < 1:
+            raise ValueError(f"streams={streams} must be at least 1")
+        self.hidden_size = int(hidden_size)
+        self.eps = float(eps)
+        self.weight_name = weight_name
+        self.streams = int(streams)
+        self.center = bool(center)
+        self.weight: Optional[torch.Tensor] = None
+
+    def params(self) -> Dict[str, Param]:
+        return {"weight": single(self.weight_name, (self.hidden_size,), role="vector", init="one_plus_normal")}
+
+    def forward_streams(self, residual, update, in_weights, ctx, rows=None):
+        """``update``: a ``StreamUpdate``, a plain delta (tensor or ``ScaledSum``: every stream takes it as it is) or None."""
+        if isinstance(update, ResidualCopy):
+            update = None
+        if update is not None and not isinstance(update, StreamUpdate):
+            update = StreamUpdate(update)
+        terms, scales = (), ()
+        if update is not None:
+            y = update.y
+            if isinstance(y, ScaledSum):
+                terms, scales = tuple(y.terms), tuple(float(s) for s in y.scales)
+            else:
+                if y.dim() == 3:
+                    y = y.sum(0)  # (float32 partial sums of a product)
+                terms, scales = (y,), (1.0,)
+        return ctx.ops.stream_norm(residual, terms, scales, update.mix if update is not None else None, update.out if update is not None else None,
+                                   in_weights, self.weight, self.eps, self.streams, self.center, ctx.dtype, rows=rows)
+
+    def forward(self, residual, delta, ctx, rows=None):
+        if isinstance(delta, DeferredNorm):
+            raise ValueError("this norm cannot be split into a product's epilogue")
+        return self.forward_streams(residual, delta, None, ctx, rows=rows)
+
+
+register_part("norm", "stream_norm", StreamNorm)

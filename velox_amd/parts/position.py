@@ -29,8 +29,12 @@ from .base import PositionEncoding, register_part
 
 class RotaryEncoding(PositionEncoding):
     def __init__(self, rotary_dim: int, theta: float, max_position: int, scaling_factor: float = 1.0, layout: str = "halves",
-                 stretch: Optional[Sequence[float]] = None) -> None:
+                 stretch: Optional[Sequence[float]] = None, exact_angles: bool = False) -> None:
+        """``exact_angles``: frequencies ``theta^(-2i/d) / scaling_factor`` and the angles ``p * f_i`` are worked out in
+        float64 and only cosine and sine are rounded to float32 (the tables then do not carry the float32 error of the
+        angle, which grows with the position)."""
         super().__init__("")
+        self.exact_angles = bool(exact_angles)
         if rotary_dim % 2 != 0:
             raise ValueError(f"rotary_dim must be even, got {rotary_dim}")
         if layout not in ("halves", "interleaved"):
@@ -65,6 +69,13 @@ class RotaryEncoding(PositionEncoding):
         return (plain / factor * ramp + plain * (1.0 - ramp)).float(), 0.1 * math.log(factor) + 1.0
 
     def finalize(self, device, dtype) -> None:
+        if self.exact_angles and self.stretch is None:
+            index = torch.arange(self.rotary_dim // 2, dtype=torch.float64)
+            freq = self.theta ** (-2.0 * index / self.rotary_dim) / self.scaling_factor
+            angles = torch.outer(torch.arange(self.max_position, dtype=torch.float64), freq)
+            self.cos = angles.cos().float().contiguous().to(device)
+            self.sin = angles.sin().float().contiguous().to(device)
+            return
         inv_freq, magnitude = self.frequencies()
         positions = torch.arange(self.max_position, dtype=torch.float32)
         if self.scaling_factor != 1.0:

@@ -33,6 +33,10 @@ def _draw(shape, init: str, generator: torch.Generator, device) -> torch.Tensor:
     values = torch.randn(tuple(shape), generator=generator, dtype=torch.float32, device=device) * _STD
     if init == "one_plus_normal":
         values = values + 1.0
+    elif init == "identity_plus_normal":  # (a square matrix near the identity)
+        values = values + torch.eye(shape[0], shape[1], dtype=torch.float32, device=device)
+    elif init == "mean_plus_normal":  # (weights of an average over the first dimension)
+        values = values + 1.0 / shape[0]
     elif init != "normal":
         raise ValueError(f"unknown init law {init!r}")
     return values
