@@ -1,0 +1,551 @@
+// Kernels of the mixers that carry a state of fixed size from token to token, and of the blocks around them, for gfx950:
+//   stream_norm         the residual streams' update (mix matrix, weighted sub-layer output) and the norm of their weighted sum
+//   gated_act_mul       act(gate) * up with the tanh form of GELU or SiLU
+//   short_conv          causal convolution over a few taps per channel, the inputs before a portion's start from the state slot
+//   rotate_pad_write    partial rotation of q and k, q at the attention kernels' head size, k and v into the paged cache
+//   recurrence_prepare  unit q and k, decay and beta of a linear recurrence, all float32
+//   linear_scan         the recurrence itself, token by token from the state slot
+//   gated_head_norm     RMS norm of each head's read-out, a shared weight, a gate
+// Everything between a load and a store is float32; stores round once.  No result depends on how a sequence's tokens
+// were cut into steps or on what else is in the batch: sums run in an order that only the sizes fix.
+#include "common.h"
+
+__device__ __forceinline__ float load_as_f32(const void* p, int is_bf16, size_t i) {
+  return is_bf16 ? to_f32(((const bf16_t*)p)[i]) : ((const float*)p)[i];
+}
+__device__ __forceinline__ void store_from_f32(void* p, int is_bf16, size_t i, float v) {
+  if (is_bf16) ((bf16_t*)p)[i] = (bf16_t)v; else ((float*)p)[i] = v;
+}
+__device__ __forceinline__ float sigmoid_f32(float z) { return 1.f / (1.f + expf(-z)); }
+__device__ __forceinline__ float softplus_f32(float z) { return z > 20.f ? z : log1pf(expf(z)); }
+
+// ---------------------------------------------------------------------------------------------
+// stream_norm.  One workgroup per output row.  residual float32 [T, S * H], stream after stream within a row.
+//   With terms: y = scale0 * term0 (+ scale1 * term1); x_t <- sum_s mix[s, t] x_s + out[t] * y for all t (mix nullptr: the
+//   identity, out nullptr: ones), written back unless `rows` picks rows.  Then u = sum_s in[s] x_s (in nullptr: ones) and
+//   out = (u - mean(u)) / sqrt(mean((u - mean)^2) + eps) * w   (center)   or   u / sqrt(mean(u^2) + eps) * w.
+//   u is kept in LDS between the passes (H floats).
+// ---------------------------------------------------------------------------------------------
+#define STREAMS_MAX 8
+struct StreamNormArgs {
+  float* residual;
+  const void* term0;
+  const void* term1;
+  int term0_bf16, term1_bf16, num_terms;
+  float scale0, scale1;
+  const float* mix;
+  const float* out_w;
+  const float* in_w;
+  const float* weight;
+  const int* rows;
+  void* out;
+  int out_bf16, hidden, streams, center;
+  float eps;
+};
+
+__global__ void __launch_bounds__(256) stream_norm_kernel(const StreamNormArgs a) {
+  extern __shared__ float u_row[];
+  __shared__ float scratch[16];
+  __shared__ float coef[STREAMS_MAX * STREAMS_MAX + 2 * STREAMS_MAX];
+  const int S = a.streams, H = a.hidden;
+  float* mix = coef;
+  float* ow = coef + STREAMS_MAX * STREAMS_MAX;
+  float* iw = ow + STREAMS_MAX;
+  if (threadIdx.x < S * S) {
+    const int s = threadIdx.x / S, t = threadIdx.x % S;
+    mix[s * STREAMS_MAX + t] = a.mix ? a.mix[s * S + t] : (s == t ? 1.f : 0.f);
+  }
+  if (threadIdx.x < S) {
+    ow[threadIdx.x] = a.out_w ? a.out_w[threadIdx.x] : 1.f;
+    iw[threadIdx.x] = a.in_w ? a.in_w[threadIdx.x] : 1.f;
+  }
+  __syncthreads();
+  const int row = blockIdx.x;
+  const size_t src = a.rows ? (size_t)a.rows[row] : (size_t)row;
+  float* res = a.residual + src * (size_t)S * H;
+  const bool update = a.num_terms > 0;
+  const bool write_back = update && a.rows == nullptr;
+  float sum = 0.f;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {
+    float x[STREAMS_MAX];
+#pragma unroll
+    for (int s = 0; s < STREAMS_MAX; ++s) x[s] = s < S ? res[(size_t)s * H + i] : 0.f;
+    float u = 0.f;
+    if (update) {
+      float y = a.scale0 * load_as_f32(a.term0, a.term0_bf16, src * H + i);
+      if (a.num_terms > 1) y += a.scale1 * load_as_f32(a.term1, a.term1_bf16, src * H + i);
+#pragma unroll
+      for (int t = 0; t < STREAMS_MAX; ++t) {
+        if (t < S) {
+          float n = 0.f;
+#pragma unroll
+          for (int s = 0; s < STREAMS_MAX; ++s)
+            if (s < S) n += mix[s * STREAMS_MAX + t] * x[s];
+          n += ow[t] * y;
+          if (write_back) res[(size_t)t * H + i] = n;
+          u += iw[t] * n;
+        }
+      }
+    } else {
+#pragma unroll
+      for (int s = 0; s < STREAMS_MAX; ++s)
+        if (s < S) u += iw[s] * x[s];
+    }
+    u_row[i] = u;
+    sum += u;
+  }
+  float mean = 0.f;
+  if (a.center) mean = block_sum(sum, scratch) / (float)H;
+  float sq = 0.f;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) {  // (each thread reads back what it wrote itself)
+    const float d = u_row[i] - mean;
+    sq += d * d;
+  }
+  const float inv = 1.f / sqrtf(block_sum(sq, scratch) / (float)H + a.eps);
+  for (int i = threadIdx.x; i < H; i += blockDim.x)
+    store_from_f32(a.out, a.out_bf16, (size_t)row * H + i, (u_row[i] - mean) * inv * a.weight[i]);
+}
+
+extern "C" int velox_stream_norm(float* residual, const void* term0, int term0_dtype, float scale0, const void* term1, int term1_dtype, float scale1,
+                                 int num_terms, const float* mix, const float* out_w, const float* in_w, const float* weight, const int* rows,
+                                 void* out, int out_dtype, int count, int hidden, int streams, int center, float eps, hipStream_t stream) {
+  if (count <= 0) return 0;
+  if (streams < 1 || streams > STREAMS_MAX || hidden < 1 || hidden > 16384 || num_terms < 0 || num_terms > 2) return (int)hipErrorInvalidValue;
+  StreamNormArgs a{residual, term0, term1, term0_dtype == VELOX_BF16, term1_dtype == VELOX_BF16, num_terms, scale0, scale1, mix, out_w, in_w, weight,
+                   rows, out, out_dtype == VELOX_BF16, hidden, streams, center, eps};
+  stream_norm_kernel<<<count, 256, (size_t)hidden * sizeof(float), stream>>>(a);
+  VELOX_RETURN_LAUNCH_STATUS();
+}
+
+// ---------------------------------------------------------------------------------------------
+// embedding written `copies` times side by side: out[t, c * H + i] = table[ids[t], i] * scale.
+// ---------------------------------------------------------------------------------------------
+__global__ void __launch_bounds__(256) embed_copies_kernel(const int* __restrict__ ids, const void* __restrict__ table, int table_bf16, float* __restrict__ out,
+                                                           int hidden, int vocab, float scale, int copies) {
+  const int t = blockIdx.x;
+  const int id = ids[t];
+  float* dst = out + (size_t)t * hidden * copies;
+  const bool ok = id >= 0 && id < vocab;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    const float v = ok ? load_as_f32(table, table_bf16, (size_t)id * hidden + i) * scale : __builtin_nanf("");
+    for (int c = 0; c < copies; ++c) dst[(size_t)c * hidden + i] = v;
+  }
+}
+
+extern "C" int velox_embed_copies(const int* ids, const void* table, int table_dtype, float* out, int tokens, int hidden, int vocab, float scale, int copies,
+                                  hipStream_t stream) {
+  if (tokens <= 0) return 0;
+  embed_copies_kernel<<<tokens, 256, 0, stream>>>(ids, table, table_dtype == VELOX_BF16, out, hidden, vocab, scale, copies);
+  VELOX_RETURN_LAUNCH_STATUS();
+}
+
+// ---------------------------------------------------------------------------------------------
+// gated_act_mul: out[t, i] = act(gate_up[t, i]) * gate_up[t, I + i]; kind 0: SiLU, 1: the tanh form of GELU.
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ float gelu_tanh_f32(float z) { return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z))); }
+
+template <typename T>
+__global__ void __launch_bounds__(256) gated_act_mul_kernel(const T* __restrict__ gate_up, T* __restrict__ out, int inter, int kind) {
+  const size_t t = blockIdx.y;
+  const T* row = gate_up + t * 2 * (size_t)inter;
+  for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < inter; i += gridDim.x * blockDim.x) {
+    const float g = to_f32(row[i]), u = to_f32(row[inter + i]);
+    const float act = kind == 1 ? gelu_tanh_f32(g) : g * sigmoid_f32(g);
+    out[t * inter + i] = from_f32<T>(act * u);
+  }
+}
+
+extern "C" int velox_gated_act_mul(const void* gate_up, void* out, int tokens, int inter, int dtype, int kind, hipStream_t stream) {
+  if (tokens <= 0 || inter <= 0) return 0;
+  if (tokens > 65535) return (int)hipErrorInvalidValue;
+  int bx = (inter + 255) / 256;
+  if (bx > 64) bx = 64;
+  const dim3 grid(bx, tokens);
+  if (dtype == VELOX_BF16) gated_act_mul_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)gate_up, (bf16_t*)out, inter, kind);
+  else gated_act_mul_kernel<float><<<grid, 256, 0, stream>>>((const float*)gate_up, (float*)out, inter, kind);
+  VELOX_RETURN_LAUNCH_STATUS();
+}
+
+// ---------------------------------------------------------------------------------------------
+// short_conv.  x [T, ld]: the first C columns pass y_t = sum_j w[c, j] u_(t - taps + 1 + j), per sequence; the inputs before a
+// portion's start are tail[slot] ([taps - 1, C], oldest first; nullptr: zeros).  Grid (channel blocks, token chunks, sequences);
+// a thread owns one channel and walks CONV_CHUNK tokens with the last taps - 1 inputs in registers.
+// The tail is brought up to date by the same thread when a sequence's portion is one chunk at most (decoding), else by
+// short_conv_tail_kernel, which runs afterwards: no workgroup writes what another still reads.
+// ---------------------------------------------------------------------------------------------
+#define CONV_TAPS_MAX 8
+#define CONV_CHUNK 16
+
+template <typename T>
+__global__ void __launch_bounds__(256) short_conv_kernel(const T* __restrict__ x, int ld, int C, const float* __restrict__ w, int taps, T* tail,
+                                                         const int* __restrict__ slots, const int* __restrict__ cu_q, T* __restrict__ out, int silu,
+                                                         int update_here) {
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  const int b = blockIdx.z;
+  const int lo = cu_q[b], hi = cu_q[b + 1];
+  const int first = lo + blockIdx.y * CONV_CHUNK;
+  if (c >= C || first >= hi) return;
+  const int last = first + CONV_CHUNK < hi ? first + CONV_CHUNK : hi;
+  float wj[CONV_TAPS_MAX], u[CONV_TAPS_MAX];
+#pragma unroll
+  for (int j = 0; j < CONV_TAPS_MAX; ++j) wj[j] = j < taps ? w[(size_t)c * taps + j] : 0.f;
+  T* my_tail = tail ? tail + (size_t)slots[b] * (taps - 1) * C + c : nullptr;
+  // u[j] is the input `taps - 1 - j` tokens before the current one; u[taps - 1] the current
+#pragma unroll
+  for (int j = 0; j < CONV_TAPS_MAX; ++j) {
+    u[j] = 0.f;
+    if (j < taps - 1) {
+      const int t = first - (taps - 1) + j;
+      if (t >= lo) u[j] = to_f32(x[(size_t)t * ld + c]);
+      else if (my_tail) u[j] = to_f32(my_tail[(size_t)(t - lo + taps - 1) * C]);
+    }
+  }
+  for (int t = first; t < last; ++t) {
+    const float now = to_f32(x[(size_t)t * ld + c]);
+    float y = 0.f;
+#pragma unroll
+    for (int j = 0; j < CONV_TAPS_MAX; ++j)  // (oldest input first; the last column of the weights meets the current token)
+      if (j < taps) y += wj[j] * (j == taps - 1 ? now : u[j]);
+    if (silu) y = y * sigmoid_f32(y);
+    out[(size_t)t * C + c] = from_f32<T>(y);
+#pragma unroll
+    for (int j = 0; j < CONV_TAPS_MAX; ++j) u[j] = j == taps - 2 ? now : (j + 1 < CONV_TAPS_MAX ? u[j + 1] : 0.f);
+  }
+  if (update_here && my_tail && taps > 1) {  // (then this thread has seen the whole portion: u[0 .. taps - 2] are the last inputs)
+#pragma unroll
+    for (int j = 0; j < CONV_TAPS_MAX; ++j)
+      if (j < taps - 1) my_tail[(size_t)j * C] = from_f32<T>(u[j]);
+  }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256) short_conv_tail_kernel(const T* __restrict__ x, int ld, int C, int taps, T* tail, const int* __restrict__ slots,
+                                                              const int* __restrict__ cu_q) {
+  const int c = blockIdx.x * blockDim.x + threadIdx.x;
+  const int b = blockIdx.y;
+  const int lo = cu_q[b], hi = cu_q[b + 1];
+  if (c >= C || hi <= lo) return;
+  T* my_tail = tail + (size_t)slots[b] * (taps - 1) * C + c;
+  float u[CONV_TAPS_MAX];
+#pragma unroll
+  for (int j = 0; j < CONV_TAPS_MAX; ++j) {
+    u[j] = 0.f;
+    if (j < taps - 1) {
+      const int t = hi - (taps - 1) + j;
+      u[j] = t >= lo ? to_f32(x[(size_t)t * ld + c]) : to_f32(my_tail[(size_t)(t - lo + taps - 1) * C]);
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < CONV_TAPS_MAX; ++j)
+    if (j < taps - 1) my_tail[(size_t)j * C] = from_f32<T>(u[j]);
+}
+
+extern "C" int velox_short_conv(const void* x, int ld, int channels, const float* w, int taps, void* tail, const int* slots, const int* cu_q, void* out,
+                                int num_seqs, int max_q_len, int dtype, int silu, int update_state, hipStream_t stream) {
+  if (num_seqs <= 0 || max_q_len <= 0) return 0;
+  if (taps < 1 || taps > CONV_TAPS_MAX || num_seqs > 65535) return (int)hipErrorInvalidValue;
+  const int chunks = (max_q_len + CONV_CHUNK - 1) / CONV_CHUNK;
+  if (chunks > 65535) return (int)hipErrorInvalidValue;
+  const dim3 grid((channels + 255) / 256, chunks, num_seqs);
+  const int here = (update_state && chunks == 1) ? 1 : 0;
+  if (dtype == VELOX_BF16)
+    short_conv_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)x, ld, channels, w, taps, (bf16_t*)tail, slots, cu_q, (bf16_t*)out, silu, here);
+  else
+    short_conv_kernel<float><<<grid, 256, 0, stream>>>((const float*)x, ld, channels, w, taps, (float*)tail, slots, cu_q, (float*)out, silu, here);
+  if (update_state && !here && tail && taps > 1) {
+    const dim3 tail_grid((channels + 255) / 256, num_seqs);
+    if (dtype == VELOX_BF16) short_conv_tail_kernel<bf16_t><<<tail_grid, 256, 0, stream>>>((const bf16_t*)x, ld, channels, taps, (bf16_t*)tail, slots, cu_q);
+    else short_conv_tail_kernel<float><<<tail_grid, 256, 0, stream>>>((const float*)x, ld, channels, taps, (float*)tail, slots, cu_q);
+  }
+  VELOX_RETURN_LAUNCH_STATUS();
+}
+
+// ---------------------------------------------------------------------------------------------
+// rotate_pad_write: one workgroup per token.  A row of qkv holds `heads` queries and `kv_heads` keys of `dim` channels and
+// `kv_heads` values of `vdim`.  The first 2 * half channels of every query and key head are rotated (channel i with i + half,
+// cos/sin float32 [positions, half]); queries go to q_out [T, heads * D], keys to k_cache [pages, kv_heads, page, D], values
+// to v_cache [pages, kv_heads, D, page]; channels from dim (vdim) to D are zeros.
+// ---------------------------------------------------------------------------------------------
+template <typename T>
+__global__ void __launch_bounds__(256) rotate_pad_write_kernel(const T* __restrict__ qkv, int ld, T* __restrict__ q_out, const int* __restrict__ positions,
+                                                               const float* __restrict__ cos_t, const float* __restrict__ sin_t, int half,
+                                                               const int* __restrict__ slot_mapping, T* __restrict__ k_cache, T* __restrict__ v_cache,
+                                                               int heads, int kv_heads, int dim, int vdim, int D, int page_shift, int write_kv) {
+  const int t = blockIdx.x;
+  const T* row = qkv + (size_t)t * ld;
+  const int q_size = heads * dim, k_size = kv_heads * dim;
+  const int page_size = 1 << page_shift;
+  int page = 0, offset = 0;
+  if (write_kv) {
+    const int slot = slot_mapping[t];
+    page = slot >> page_shift;
+    offset = slot & (page_size - 1);
+  }
+  const float* cs = half > 0 ? cos_t + (size_t)positions[t] * half : nullptr;
+  const float* sn = half > 0 ? sin_t + (size_t)positions[t] * half : nullptr;
+  const int all = (heads + (write_kv ? kv_heads : 0)) * D;
+  for (int i = threadIdx.x; i < all; i += blockDim.x) {
+    const int h = i / D, c = i % D;
+    const bool is_q = h < heads;
+    const int g = is_q ? h : h - heads;
+    const T* src = row + (is_q ? h * dim : q_size + g * dim);
+    float v = 0.f;
+    if (c < dim) {
+      v = to_f32(src[c]);
+      if (c < half) v = v * cs[c] - to_f32(src[c + half]) * sn[c];
+      else if (c < 2 * half) v = v * cs[c - half] + to_f32(src[c - half]) * sn[c - half];
+    }
+    T* dst = is_q ? q_out + ((size_t)t * heads + h) * D : k_cache + (((size_t)page * kv_heads + g) * page_size + offset) * D;
+    dst[c] = from_f32<T>(v);
+  }
+  if (!write_kv) return;
+  const T* values = row + q_size + k_size;
+  for (int i = threadIdx.x; i < kv_heads * D; i += blockDim.x) {
+    const int g = i / D, c = i % D;
+    v_cache[(((size_t)page * kv_heads + g) * D + c) * page_size + offset] = c < vdim ? values[g * vdim + c] : from_f32<T>(0.f);
+  }
+}
+
+extern "C" int velox_rotate_pad_write(const void* qkv, int ld, void* q_out, const int* positions, const float* cos_t, const float* sin_t, int half,
+                                      const int* slot_mapping, void* k_cache, void* v_cache, int tokens, int heads, int kv_heads, int dim, int vdim, int D,
+                                      int page_size, int write_kv, int dtype, hipStream_t stream) {
+  if (tokens <= 0) return 0;
+  int shift = 0;
+  while ((1 << shift) < page_size) ++shift;
+  if ((1 << shift) != page_size || 2 * half > dim || dim > D || vdim > D) return (int)hipErrorInvalidValue;
+  if (dtype == VELOX_BF16)
+    rotate_pad_write_kernel<bf16_t><<<tokens, 256, 0, stream>>>((const bf16_t*)qkv, ld, (bf16_t*)q_out, positions, cos_t, sin_t, half, slot_mapping,
+                                                                (bf16_t*)k_cache, (bf16_t*)v_cache, heads, kv_heads, dim, vdim, D, shift, write_kv);
+  else
+    rotate_pad_write_kernel<float><<<tokens, 256, 0, stream>>>((const float*)qkv, ld, (float*)q_out, positions, cos_t, sin_t, half, slot_mapping,
+                                                               (float*)k_cache, (float*)v_cache, heads, kv_heads, dim, vdim, D, shift, write_kv);
+  VELOX_RETURN_LAUNCH_STATUS();
+}
+
+// ---------------------------------------------------------------------------------------------
+// recurrence_prepare: one workgroup per token, waves take heads in turn.
+//   qk float32 [T, kv_heads, 2, dim]: q (unit vector if `unit`, times q_scale), then k (unit vector if `unit`);
+//   decay float32 [T, columns] = exp(-rate[h] * softplus(sign * (z + bias))), h = column / (columns / heads);
+//   beta float32 [T, heads] = sigmoid(b).
+// ---------------------------------------------------------------------------------------------
+struct PrepareArgs {
+  const void* qkv;
+  int qkv_bf16, ld, q_at, k_at, kv_heads, dim, unit;
+  float q_scale;
+  const void* decay_src;
+  int decay_bf16, decay_ld, decay_at, heads, columns;
+  const float* rate;
+  const float* bias;
+  float sign;
+  const void* beta_src;
+  int beta_bf16, beta_ld, beta_at;
+  float* qk;
+  float* decay;
+  float* beta;
+};
+
+__global__ void __launch_bounds__(256) recurrence_prepare_kernel(const PrepareArgs a) {
+  const size_t t = blockIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (int h = wave; h < 2 * a.kv_heads; h += 4) {
+    const int g = h >> 1, is_k = h & 1;
+    const size_t at = t * a.ld + (is_k ? a.k_at : a.q_at) + (size_t)g * a.dim;
+    float inv = 1.f;
+    if (a.unit) {
+      float s = 0.f;
+      for (int c = lane; c < a.dim; c += 64) { const float v = load_as_f32(a.qkv, a.qkv_bf16, at + c); s += v * v; }
+      s = wave_sum(s);
+      inv = 1.f / sqrtf(s + 1e-6f);
+    }
+    const float factor = is_k ? 1.f : a.q_scale;
+    float* dst = a.qk + ((t * a.kv_heads + g) * 2 + is_k) * a.dim;
+    for (int c = lane; c < a.dim; c += 64) dst[c] = load_as_f32(a.qkv, a.qkv_bf16, at + c) * inv * factor;
+  }
+  const int per_head = a.columns / a.heads;
+  for (int c = threadIdx.x; c < a.columns; c += blockDim.x) {
+    float z = load_as_f32(a.decay_src, a.decay_bf16, t * a.decay_ld + a.decay_at + c);
+    if (a.bias) z += a.bias[c];
+    a.decay[t * a.columns + c] = expf(-a.rate[c / per_head] * softplus_f32(a.sign * z));
+  }
+  if (a.beta)
+    for (int h = threadIdx.x; h < a.heads; h += blockDim.x)
+      a.beta[t * a.heads + h] = sigmoid_f32(load_as_f32(a.beta_src, a.beta_bf16, t * a.beta_ld + a.beta_at + h));
+}
+
+extern "C" int velox_recurrence_prepare(const void* qkv, int qkv_dtype, int ld, int q_at, int k_at, int kv_heads, int dim, int unit, float q_scale,
+                                        const void* decay_src, int decay_dtype, int decay_ld, int decay_at, int heads, int columns, const float* rate,
+                                        const float* bias, float sign, const void* beta_src, int beta_dtype, int beta_ld, int beta_at, float* qk,
+                                        float* decay, float* beta, int tokens, hipStream_t stream) {
+  if (tokens <= 0) return 0;
+  if (heads < 1 || columns % heads != 0) return (int)hipErrorInvalidValue;
+  PrepareArgs a{qkv, qkv_dtype == VELOX_BF16, ld, q_at, k_at, kv_heads, dim, unit, q_scale, decay_src, decay_dtype == VELOX_BF16, decay_ld, decay_at, heads,
+                columns, rate, bias, sign, beta_src, beta_dtype == VELOX_BF16, beta_ld, beta_at, qk, decay, beta};
+  recurrence_prepare_kernel<<<tokens, 256, 0, stream>>>(a);
+  VELOX_RETURN_LAUNCH_STATUS();
+}
+
+// ---------------------------------------------------------------------------------------------
+// linear_scan.  Per sequence and head a state S of dim x vdim float32 numbers (rows: key channels) in state[slot, head].
+// Every column of S is a recurrence of its own:   s <- g * s;  u = beta (v_e - k . s)  (delta rule)  or  u = v_e;
+// s <- s + k u;  o_e = q . s.   A column is held by R lanes of a wave, SCAN_ROWS consecutive rows each (R the smallest power of
+// two with R * SCAN_ROWS >= dim: a function of dim alone, so the order of every sum is too); the two dot products are
+// reduced over those lanes.  The next token's q, k, decay, value and beta are loaded while the current one is worked on.
+// Grid (column blocks, heads, sequences); a workgroup of 256 lanes holds 256 / R columns.
+// ---------------------------------------------------------------------------------------------
+#define SCAN_ROWS 16
+
+struct ScanArgs {
+  const float* qk;       // [T, kv_heads, 2, dim]
+  const void* v;         // [T, v_ld], a token's values at v_at
+  int v_bf16, v_ld, v_at;
+  const float* decay;    // [T, heads * dim] or [T, heads]
+  int decay_per_channel;
+  const float* beta;     // [T, heads] or nullptr
+  float* state;          // [slots, heads, dim, vdim]
+  const int* slots;
+  const int* cu_q;
+  float* out;            // [T, heads * vdim]
+  int heads, kv_heads, dim, vdim, delta;
+};
+
+__device__ __forceinline__ void scan_load_rows(const float* __restrict__ p, int d0, int dim, bool vec, float fill, float (&r)[SCAN_ROWS]) {
+  if (vec && d0 + SCAN_ROWS <= dim) {
+#pragma unroll
+    for (int i = 0; i < SCAN_ROWS; i += 4) {
+      const float4_t x = *reinterpret_cast<const float4_t*>(p + d0 + i);
+      r[i] = x[0]; r[i + 1] = x[1]; r[i + 2] = x[2]; r[i + 3] = x[3];
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < SCAN_ROWS; ++i) r[i] = d0 + i < dim ? p[d0 + i] : fill;
+  }
+}
+
+template <int R>
+__global__ void __launch_bounds__(256) linear_scan_kernel(const ScanArgs a) {
+  const int r = threadIdx.x % R;
+  const int e = blockIdx.x * (256 / R) + threadIdx.x / R;
+  const int h = blockIdx.y, b = blockIdx.z;
+  const int lo = a.cu_q[b], hi = a.cu_q[b + 1];
+  if (hi <= lo) return;
+  const bool live = e < a.vdim;
+  const int col = live ? e : a.vdim - 1;  // (lanes beyond the last column follow it and write nothing: the shuffles need every lane)
+  const int dim = a.dim, vdim = a.vdim;
+  const int d0 = r * SCAN_ROWS;
+  const int g = h / (a.heads / a.kv_heads);
+  const bool vec = (dim % 4) == 0;
+  float* S = a.state + (((size_t)a.slots[b] * a.heads + h) * dim) * vdim + col;
+  float s[SCAN_ROWS];
+#pragma unroll
+  for (int i = 0; i < SCAN_ROWS; ++i) s[i] = d0 + i < dim ? S[(size_t)(d0 + i) * vdim] : 0.f;
+
+  float q[SCAN_ROWS], k[SCAN_ROWS], dec[SCAN_ROWS], qn[SCAN_ROWS], kn[SCAN_ROWS], decn[SCAN_ROWS];
+  float val, bet, valn = 0.f, betn = 1.f;
+  auto fetch = [&](int t, float (&fq)[SCAN_ROWS], float (&fk)[SCAN_ROWS], float (&fd)[SCAN_ROWS], float& fv, float& fb) {
+    const float* base = a.qk + ((size_t)t * a.kv_heads + g) * 2 * dim;
+    scan_load_rows(base, d0, dim, vec, 0.f, fq);
+    scan_load_rows(base + dim, d0, dim, vec, 0.f, fk);
+    if (a.decay_per_channel) {
+      scan_load_rows(a.decay + ((size_t)t * a.heads + h) * dim, d0, dim, vec, 1.f, fd);
+    } else {
+      const float one = a.decay[(size_t)t * a.heads + h];
+#pragma unroll
+      for (int i = 0; i < SCAN_ROWS; ++i) fd[i] = one;
+    }
+    fv = load_as_f32(a.v, a.v_bf16, (size_t)t * a.v_ld + a.v_at + (size_t)h * vdim + col);
+    fb = a.beta ? a.beta[(size_t)t * a.heads + h] : 1.f;
+  };
+  fetch(lo, q, k, dec, val, bet);
+  for (int t = lo; t < hi; ++t) {
+    if (t + 1 < hi) fetch(t + 1, qn, kn, decn, valn, betn);
+    float dot = 0.f;
+#pragma unroll
+    for (int i = 0; i < SCAN_ROWS; ++i) {
+      s[i] *= dec[i];
+      dot += s[i] * k[i];
+    }
+    float u = val;
+    if (a.delta) {
+#pragma unroll
+      for (int off = 1; off < R; off <<= 1) dot += __shfl_xor(dot, off, VELOX_WAVE);
+      u = bet * (val - dot);
+    }
+    float o = 0.f;
+#pragma unroll
+    for (int i = 0; i < SCAN_ROWS; ++i) {
+      s[i] += k[i] * u;
+      o += s[i] * q[i];
+    }
+#pragma unroll
+    for (int off = 1; off < R; off <<= 1) o += __shfl_xor(o, off, VELOX_WAVE);
+    if (live && r == 0) a.out[((size_t)t * a.heads + h) * vdim + e] = o;
+#pragma unroll
+    for (int i = 0; i < SCAN_ROWS; ++i) { q[i] = qn[i]; k[i] = kn[i]; dec[i] = decn[i]; }
+    val = valn; bet = betn;
+  }
+  if (live) {
+#pragma unroll
+    for (int i = 0; i < SCAN_ROWS; ++i)
+      if (d0 + i < dim) S[(size_t)(d0 + i) * vdim] = s[i];
+  }
+}
+
+extern "C" int velox_linear_scan_lanes(int dim) {
+  int lanes = 1;
+  while (lanes * SCAN_ROWS < dim) lanes <<= 1;
+  return lanes;
+}
+
+extern "C" int velox_linear_scan(const float* qk, const void* v, int v_dtype, int v_ld, int v_at, const float* decay, int decay_per_channel, const float* beta,
+                                 float* state, const int* slots, const int* cu_q, float* out, int num_seqs, int heads, int kv_heads, int dim, int vdim,
+                                 int delta, hipStream_t stream) {
+  if (num_seqs <= 0) return 0;
+  const int lanes = velox_linear_scan_lanes(dim);
+  if (lanes > 64 || heads > 65535 || num_seqs > 65535 || kv_heads < 1 || heads % kv_heads != 0 || (delta && !beta)) return (int)hipErrorInvalidValue;
+  ScanArgs a{qk, v, v_dtype == VELOX_BF16, v_ld, v_at, decay, decay_per_channel, beta, state, slots, cu_q, out, heads, kv_heads, dim, vdim, delta};
+  const int cols = 256 / lanes;
+  const dim3 grid((vdim + cols - 1) / cols, heads, num_seqs);
+  switch (lanes) {
+    case 1: linear_scan_kernel<1><<<grid, 256, 0, stream>>>(a); break;
+    case 2: linear_scan_kernel<2><<<grid, 256, 0, stream>>>(a); break;
+    case 4: linear_scan_kernel<4><<<grid, 256, 0, stream>>>(a); break;
+    case 8: linear_scan_kernel<8><<<grid, 256, 0, stream>>>(a); break;
+    case 16: linear_scan_kernel<16><<<grid, 256, 0, stream>>>(a); break;
+    case 32: linear_scan_kernel<32><<<grid, 256, 0, stream>>>(a); break;
+    default: linear_scan_kernel<64><<<grid, 256, 0, stream>>>(a); break;
+  }
+  VELOX_RETURN_LAUNCH_STATUS();
+}
+
+// ---------------------------------------------------------------------------------------------
+// gated_head_norm: one wave per (token, head): out = o / sqrt(mean(o^2) + eps) * w * gate, gate = silu(z) (kind 0) or
+// sigmoid(z) (kind 1), z a token's row of gate_src at gate_at.
+// ---------------------------------------------------------------------------------------------
+__global__ void __launch_bounds__(256) gated_head_norm_kernel(const float* __restrict__ read, const float* __restrict__ weight, float eps,
+                                                              const void* __restrict__ gate_src, int gate_bf16, int gate_ld, int gate_at, int kind,
+                                                              void* __restrict__ out, int out_bf16, int heads, int vdim, size_t pairs) {
+  const size_t pair = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (pair >= pairs) return;
+  const int lane = threadIdx.x & 63;
+  const size_t t = pair / heads;
+  const int h = (int)(pair % heads);
+  const float* o = read + pair * vdim;
+  float s = 0.f;
+  for (int c = lane; c < vdim; c += 64) s += o[c] * o[c];
+  s = wave_sum(s);
+  const float inv = 1.f / sqrtf(s / (float)vdim + eps);
+  for (int c = lane; c < vdim; c += 64) {
+    const float z = load_as_f32(gate_src, gate_bf16, t * gate_ld + gate_at + (size_t)h * vdim + c);
+    const float gate = kind == 0 ? z * sigmoid_f32(z) : sigmoid_f32(z);
+    store_from_f32(out, out_bf16, pair * vdim + c, o[c] * inv * weight[c] * gate);
+  }
+}
+
+extern "C" int velox_gated_head_norm(const float* read, const float* weight, float eps, const void* gate_src, int gate_dtype, int gate_ld, int gate_at,
+                                     int kind, void* out, int out_dtype, int tokens, int heads, int vdim, hipStream_t stream) {
+  if (tokens <= 0) return 0;
+  const size_t pairs = (size_t)tokens * heads;
+  gated_head_norm_kernel<<<(unsigned)((pairs + 3) / 4), 256, 0, stream>>>(read, weight, eps, gate_src, gate_dtype == VELOX_BF16, gate_ld, gate_at, kind, out,
+                                                                         out_dtype == VELOX_BF16, heads, vdim, pairs);
+  VELOX_RETURN_LAUNCH_STATUS();
+}

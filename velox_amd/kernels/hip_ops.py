@@ -158,6 +158,18 @@ class HipOps:
         c.velox_add_cast.argtypes = [_P, _P, _I, _P, ctypes.c_longlong, _P]
         c.velox_norm_add.argtypes = [_P, _P, _I, _P, _P, _I, _I, _F, _F, _I, ctypes.c_longlong, _P]
         c.velox_qk_norm_write.argtypes = [_P, _I, _P, _P, _P, _P, _P, _I, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _F, _F, _I, _I, _P]
+        c.velox_stream_norm.argtypes = [_P, _P, _I, _F, _P, _I, _F, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _F, _P]
+        c.velox_embed_copies.argtypes = [_P, _P, _I, _P, _I, _I, _I, _F, _I, _P]
+        c.velox_gated_act_mul.argtypes = [_P, _P, _I, _I, _I, _I, _P]
+        c.velox_short_conv.argtypes = [_P, _I, _I, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P]
+        c.velox_rotate_pad_write.argtypes = [_P, _I, _P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P]
+        c.velox_recurrence_prepare.argtypes = [_P, _I, _I, _I, _I, _I, _I, _I, _F, _P, _I, _I, _I, _I, _I, _P, _P, _F, _P, _I, _I, _I, _P, _P, _P, _I, _P]
+        c.velox_linear_scan.argtypes = [_P, _P, _I, _I, _I, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P]
+        c.velox_linear_scan_lanes.argtypes = [_I]
+        c.velox_gated_head_norm.argtypes = [_P, _P, _F, _P, _I, _I, _I, _I, _P, _I, _I, _I, _I, _P]
+        for fn in (c.velox_stream_norm, c.velox_embed_copies, c.velox_gated_act_mul, c.velox_short_conv, c.velox_rotate_pad_write, c.velox_recurrence_prepare,
+                   c.velox_linear_scan, c.velox_linear_scan_lanes, c.velox_gated_head_norm):
+            fn.restype = _I
         c.velox_routed_products_bf16.restype = _I
         for fn in (c.velox_latent_rotate_write, c.velox_head_linear, c.velox_route_top, c.velox_routed_plan, c.velox_grouped_glu, c.velox_grouped_down,
                    c.velox_routed_combine, c.velox_add_sinusoid, c.velox_add_cast, c.velox_norm_add, c.velox_qk_norm_write):
@@ -316,12 +328,20 @@ class HipOps:
             raise KernelError(f"{what}: launch failed with HIP error {status}")
 
     # -- embedding and norms ----------------------------------------------------------------------
-    def embed(self, token_ids: torch.Tensor, table: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
+    def embed(self, token_ids: torch.Tensor, table: torch.Tensor, scale: float = 1.0, copies: int = 1) -> torch.Tensor:
+        """``copies`` > 1: every row is written that many times side by side, ``[T, copies * H]`` (residual streams)."""
         self._check("token_ids", token_ids, torch.int32)
         self._check("table", table)
         if token_ids.dim() != 1 or table.dim() != 2:
             raise KernelError("embed: token_ids must be [T] and the table [V, H]")
         vocab, hidden = table.shape
+        if copies != 1:
+            if copies < 1:
+                raise KernelError(f"embed: copies={copies} must be at least 1")
+            out = torch.empty((token_ids.shape[0], copies * hidden), dtype=torch.float32, device=self.device)
+            self._launched(self._core.velox_embed_copies(_ptr(token_ids), _ptr(table), _code(table.dtype), _ptr(out), token_ids.shape[0], hidden, vocab,
+                                                         float(scale), int(copies), self._stream()), "embed")
+            return out
         out = torch.empty((token_ids.shape[0], hidden), dtype=torch.float32, device=self.device)
         status = self._core.velox_embed(_ptr(token_ids), _ptr(table), _ptr(out), token_ids.shape[0], hidden, vocab, _code(table.dtype), float(scale), self._stream())
         self._launched(status, "embed")
@@ -733,6 +753,202 @@ class HipOps:
         out = torch.empty((tokens, inter), dtype=gate_up.dtype, device=self.device)
         status = self._core.velox_silu_mul(_ptr(gate_up), _ptr(out), tokens, inter, _code(gate_up.dtype), self._stream())
         self._launched(status, "silu_mul")
+        return out
+
+    # -- residual streams, short convolution, linear recurrences ------------------------------------
+    MAX_STREAMS = 8
+    MAX_STREAM_WIDTH = 16384
+    MAX_CONV_TAPS = 8
+
+    def stream_norm(self, residual, terms, scales, mix, out_weights, in_weights, weight, eps, streams, center, out_dtype, rows=None):
+        """``residual`` float32 ``[T, streams * H]``.  With ``terms`` (one or two ``[T, H]`` tensors, ``y = sum_i scales[i] terms[i]``):
+        ``x_t <- sum_s mix[s, t] x_s + out_weights[t] y`` for all streams at once (``mix`` None: the identity, ``out_weights``
+        None: ones), in place unless ``rows`` picks rows.  Returns ``norm(sum_s in_weights[s] x_s) * weight`` in
+        ``out_dtype``, for all rows or for ``rows``; ``center``: a layer norm without bias, else an RMS norm."""
+        self._check("residual", residual, torch.float32)
+        if residual.dim() != 2 or streams < 1 or residual.shape[1] % streams != 0:
+            raise KernelError(f"stream_norm: residual must be [T, streams * H], got {tuple(residual.shape)} for {streams} streams")
+        tokens, hidden = residual.shape[0], residual.shape[1] // streams
+        if streams > self.MAX_STREAMS or hidden > self.MAX_STREAM_WIDTH:
+            raise KernelError(f"stream_norm: at most {self.MAX_STREAMS} streams of at most {self.MAX_STREAM_WIDTH} channels")
+        self._check("weight", weight, torch.float32, (hidden,))
+        if len(terms) > 2 or len(terms) != len(scales):
+            raise KernelError("stream_norm: one or two terms, each with its scale")
+        for i, term in enumerate(terms):
+            self._check(f"term {i}", term, None, (tokens, hidden))
+        for name, t, shape in (("mix", mix, (streams, streams)), ("out_weights", out_weights, (streams,)), ("in_weights", in_weights, (streams,))):
+            if t is not None:
+                self._check(name, t, torch.float32, shape)
+        if rows is not None:
+            self._check("rows", rows, torch.int32)
+        count = tokens if rows is None else rows.shape[0]
+        out = torch.empty((count, hidden), dtype=out_dtype, device=self.device)
+        t0 = terms[0] if len(terms) > 0 else None
+        t1 = terms[1] if len(terms) > 1 else None
+        status = self._core.velox_stream_norm(
+            _ptr(residual), _ptr(t0), _code(t0.dtype) if t0 is not None else 0, float(scales[0]) if t0 is not None else 0.0,
+            _ptr(t1), _code(t1.dtype) if t1 is not None else 0, float(scales[1]) if t1 is not None else 0.0, len(terms),
+            _ptr(mix), _ptr(out_weights), _ptr(in_weights), _ptr(weight), _ptr(rows), _ptr(out), _code(out_dtype), count, hidden, int(streams),
+            int(bool(center)), float(eps), self._stream())
+        self._launched(status, "stream_norm")
+        return out
+
+    def gated_act_mul(self, gate_up: torch.Tensor, activation: str) -> torch.Tensor:
+        """``act(gate) * up`` of ``[T, 2 * I]`` (gate first), ``activation`` ``"silu"`` or ``"gelu_tanh"``; float32 inside."""
+        self._check("gate_up", gate_up)
+        kinds = {"silu": 0, "gelu_tanh": 1}
+        if gate_up.dim() != 2 or gate_up.shape[1] % 2 != 0 or activation not in kinds:
+            raise KernelError("gated_act_mul: expected [T, 2 * intermediate] and 'silu' or 'gelu_tanh'")
+        tokens, inter = gate_up.shape[0], gate_up.shape[1] // 2
+        out = torch.empty((tokens, inter), dtype=gate_up.dtype, device=self.device)
+        for first in range(0, tokens, 65535):
+            count = min(65535, tokens - first)
+            self._launched(self._core.velox_gated_act_mul(_ptr(gate_up[first:first + count]), _ptr(out[first:first + count]), count, inter,
+                                                          _code(gate_up.dtype), kinds[activation], self._stream()), "gated_act_mul")
+        return out
+
+    def short_conv(self, x, channels, weight, tail, slots, cu_q, max_q_len, activation="none", update_state=True):
+        """The first ``channels`` columns of ``x`` [T, >= channels] through ``y_t = sum_j w[:, j] u_(t - taps + 1 + j)`` per sequence
+        (``weight`` float32 [channels, taps]); the inputs before a portion's start come from ``tail[slot]`` ([taps - 1, channels],
+        oldest first, the dtype of ``x``; None: zeros), which is brought up to date unless ``update_state`` is false.
+        ``activation``: ``"none"`` or ``"silu"``.  Returns [T, channels] in x's dtype."""
+        self._check("x", x)
+        if x.dim() != 2 or x.shape[1] < channels:
+            raise KernelError(f"short_conv: x {tuple(x.shape)} has fewer than {channels} columns")
+        if weight.dim() != 2:
+            raise KernelError("short_conv: the weights must be [channels, taps]")
+        taps = weight.shape[1]
+        self._check("weight", weight, torch.float32, (channels, taps))
+        if not 1 <= taps <= self.MAX_CONV_TAPS:
+            raise KernelError(f"short_conv: 1 to {self.MAX_CONV_TAPS} taps, got {taps}")
+        self._check("slots", slots, torch.int32)
+        self._check("cu_q", cu_q, torch.int32, (slots.shape[0] + 1,))
+        if tail is not None and taps > 1:
+            self._check("tail", tail, x.dtype)
+            if tail.dim() != 3 or tuple(tail.shape[1:]) != (taps - 1, channels):
+                raise KernelError(f"short_conv: the state must be [slots, {taps - 1}, {channels}], got {tuple(tail.shape)}")
+        else:
+            tail = None
+        if activation not in ("none", "silu"):
+            raise KernelError(f"short_conv: activation {activation!r}")
+        out = torch.empty((x.shape[0], channels), dtype=x.dtype, device=self.device)
+        status = self._core.velox_short_conv(_ptr(x), x.shape[1], int(channels), _ptr(weight), taps, _ptr(tail), _ptr(slots), _ptr(cu_q), _ptr(out),
+                                             slots.shape[0], int(max_q_len), _code(x.dtype), int(activation == "silu"), int(bool(update_state)), self._stream())
+        self._launched(status, "short_conv")
+        return out
+
+    def rotate_pad_write(self, qkv, num_heads, num_kv_heads, dim, vdim, cached_dim, positions, cos, sin, slot_mapping, k_cache, v_cache, block_size, write_kv=True):
+        """Rotates the first ``2 * cos.shape[1]`` channels of every q and k head of ``qkv`` [T, heads * dim + kv_heads * (dim + vdim)]
+        (channel i with i + half), writes k and v into the pages at ``cached_dim`` channels a head (zeros in the padding)
+        and returns q as [T, heads * cached_dim]."""
+        self._check("qkv", qkv)
+        tokens = qkv.shape[0]
+        width = num_heads * dim + num_kv_heads * (dim + vdim)
+        if qkv.dim() != 2 or qkv.shape[1] != width:
+            raise KernelError(f"rotate_pad_write: qkv must be [T, {width}], got {tuple(qkv.shape)}")
+        if dim > cached_dim or vdim > cached_dim:
+            raise KernelError("rotate_pad_write: the cached head size must cover dim and vdim")
+        self._check("positions", positions, torch.int32, (tokens,))
+        half = 0
+        if cos is not None:
+            half = cos.shape[1]
+            self._check("cos", cos, torch.float32)
+            self._check("sin", sin, torch.float32, tuple(cos.shape))
+            if 2 * half > dim:
+                raise KernelError(f"rotate_pad_write: the rotation spans {2 * half} channels of heads of {dim}")
+        if write_kv:
+            self._check("slot_mapping", slot_mapping, torch.int32, (tokens,))
+            self._check("k_cache", k_cache, qkv.dtype)
+            self._check("v_cache", v_cache, qkv.dtype)
+            if tuple(k_cache.shape[1:]) != (num_kv_heads, block_size, cached_dim) or tuple(v_cache.shape[1:]) != (num_kv_heads, cached_dim, block_size):
+                raise KernelError(f"rotate_pad_write: pages of {tuple(k_cache.shape[1:])} / {tuple(v_cache.shape[1:])} do not hold "
+                                  f"{num_kv_heads} heads of {cached_dim} over {block_size} tokens")
+        q = torch.empty((tokens, num_heads * cached_dim), dtype=qkv.dtype, device=self.device)
+        status = self._core.velox_rotate_pad_write(_ptr(qkv), width, _ptr(q), _ptr(positions), _ptr(cos), _ptr(sin), half, _ptr(slot_mapping) if write_kv else _P(0),
+                                                   _ptr(k_cache) if write_kv else _P(0), _ptr(v_cache) if write_kv else _P(0), tokens, num_heads, num_kv_heads,
+                                                   dim, vdim, cached_dim, int(block_size), int(bool(write_kv)), _code(qkv.dtype), self._stream())
+        self._launched(status, "rotate_pad_write")
+        return q
+
+    def recurrence_prepare(self, qkv, q_at, k_at, kv_heads, dim, unit, q_scale, decay_source, decay_at, heads, decay_columns, rate, bias, sign,
+                           beta_source, beta_at):
+        """-> ``qk`` float32 [T, kv_heads, 2, dim] (a head's q, unit vector if ``unit``, times ``q_scale``; then its k), ``decay``
+        float32 [T, decay_columns] = ``exp(-rate[h] softplus(sign (z + bias)))``, ``beta`` float32 [T, heads] = ``sigmoid(b)`` or None."""
+        self._check("qkv", qkv)
+        tokens = qkv.shape[0]
+        if qkv.dim() != 2 or max(q_at, k_at) + kv_heads * dim > qkv.shape[1]:
+            raise KernelError("recurrence_prepare: q and k do not lie within the rows of qkv")
+        self._check("decay_source", decay_source)
+        if decay_source.dim() != 2 or decay_source.shape[0] != tokens or decay_at + decay_columns > decay_source.shape[1] or decay_columns % heads != 0:
+            raise KernelError("recurrence_prepare: the decay's columns do not lie within its source")
+        self._check("rate", rate, torch.float32, (heads,))
+        if bias is not None:
+            self._check("bias", bias, torch.float32, (decay_columns,))
+        beta = None
+        if beta_source is not None:
+            self._check("beta_source", beta_source)
+            if beta_source.dim() != 2 or beta_source.shape[0] != tokens or beta_at + heads > beta_source.shape[1]:
+                raise KernelError("recurrence_prepare: beta's columns do not lie within its source")
+            beta = torch.empty((tokens, heads), dtype=torch.float32, device=self.device)
+        qk = torch.empty((tokens, kv_heads, 2, dim), dtype=torch.float32, device=self.device)
+        decay = torch.empty((tokens, decay_columns), dtype=torch.float32, device=self.device)
+        status = self._core.velox_recurrence_prepare(
+            _ptr(qkv), _code(qkv.dtype), qkv.shape[1], int(q_at), int(k_at), int(kv_heads), int(dim), int(bool(unit)), float(q_scale),
+            _ptr(decay_source), _code(decay_source.dtype), decay_source.shape[1], int(decay_at), int(heads), int(decay_columns), _ptr(rate), _ptr(bias), float(sign),
+            _ptr(beta_source), _code(beta_source.dtype) if beta_source is not None else 0, beta_source.shape[1] if beta_source is not None else 0, int(beta_at),
+            _ptr(qk), _ptr(decay), _ptr(beta), tokens, self._stream())
+        self._launched(status, "recurrence_prepare")
+        return qk, decay, beta
+
+    def linear_scan_supports(self, dim: int, vdim: int) -> None:
+        """Raises if the scan kernel cannot hold a column of a ``dim x vdim`` state in one wave."""
+        if self._core.velox_linear_scan_lanes(int(dim)) > 64:
+            raise KernelError(f"linear_scan: key heads of {dim} channels are beyond the kernel (1024 at most)")
+
+    def linear_scan(self, qk, v_source, v_at, decay, beta, state, slots, cu_q, max_q_len, heads, kv_heads, dim, vdim, delta):
+        """Per sequence and head, token by token from ``state[slot, head]`` ([dim, vdim] float32), which is written back:
+        ``S <- g S`` (rows); ``u = beta (v - S^T k)`` (``delta``) or ``u = v``; ``S <- S + k u^T``; ``o = S^T q``.  ``decay`` is
+        [T, heads] or [T, heads * dim].  Returns float32 [T, heads * vdim]."""
+        tokens = qk.shape[0]
+        self._check("qk", qk, torch.float32, (tokens, kv_heads, 2, dim), align=16)
+        self._check("v_source", v_source)
+        if v_source.dim() != 2 or v_source.shape[0] != tokens or v_at + heads * vdim > v_source.shape[1]:
+            raise KernelError("linear_scan: the values do not lie within their source")
+        self._check("decay", decay, torch.float32, align=16)
+        if tuple(decay.shape) not in ((tokens, heads), (tokens, heads * dim)):
+            raise KernelError(f"linear_scan: decay must be [T, heads] or [T, heads * dim], got {tuple(decay.shape)}")
+        per_channel = tuple(decay.shape) == (tokens, heads * dim)
+        if delta:
+            if beta is None:
+                raise KernelError("linear_scan: the delta rule needs beta")
+            self._check("beta", beta, torch.float32, (tokens, heads))
+        self._check("state", state, torch.float32)
+        if state.dim() != 4 or tuple(state.shape[1:]) != (heads, dim, vdim):
+            raise KernelError(f"linear_scan: the state must be [slots, {heads}, {dim}, {vdim}], got {tuple(state.shape)}")
+        self._check("slots", slots, torch.int32)
+        self._check("cu_q", cu_q, torch.int32, (slots.shape[0] + 1,))
+        self.linear_scan_supports(dim, vdim)
+        out = torch.empty((tokens, heads * vdim), dtype=torch.float32, device=self.device)
+        status = self._core.velox_linear_scan(_ptr(qk), _ptr(v_source), _code(v_source.dtype), v_source.shape[1], int(v_at), _ptr(decay), int(per_channel),
+                                              _ptr(beta) if delta else _P(0), _ptr(state), _ptr(slots), _ptr(cu_q), _ptr(out), slots.shape[0], int(heads),
+                                              int(kv_heads), int(dim), int(vdim), int(bool(delta)), self._stream())
+        self._launched(status, "linear_scan")
+        return out
+
+    def gated_head_norm(self, read, weight, eps, gate_source, gate_at, gate_kind, heads, vdim, out_dtype):
+        """``read`` float32 [T, heads * vdim]: every head divided by its root mean square (``eps`` inside the root), times
+        ``weight`` [vdim], times ``silu(z)`` or ``sigmoid(z)`` of the gate's columns; [T, heads * vdim] in ``out_dtype``."""
+        tokens = read.shape[0]
+        self._check("read", read, torch.float32, (tokens, heads * vdim))
+        self._check("weight", weight, torch.float32, (vdim,))
+        self._check("gate_source", gate_source)
+        if gate_source.dim() != 2 or gate_source.shape[0] != tokens or gate_at + heads * vdim > gate_source.shape[1] or gate_kind not in ("silu", "sigmoid"):
+            raise KernelError("gated_head_norm: the gate's columns do not lie within its source, or its kind is unknown")
+        out = torch.empty((tokens, heads * vdim), dtype=out_dtype, device=self.device)
+        status = self._core.velox_gated_head_norm(_ptr(read), _ptr(weight), float(eps), _ptr(gate_source), _code(gate_source.dtype), gate_source.shape[1],
+                                                  int(gate_at), 0 if gate_kind == "silu" else 1, _ptr(out), _code(out_dtype), tokens, int(heads), int(vdim),
+                                                  self._stream())
+        self._launched(status, "gated_head_norm")
         return out
 
     # -- rotary + cache write ---------------------------------------------------------------------
