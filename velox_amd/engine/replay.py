@@ -100,9 +100,10 @@ class Replayer:
         return logits.float().cpu().numpy().astype("<f4", copy=False)
 
 
-def run(model_dir: str, dtype: str, out_dir: str, max_tokens: int, block_size: int = 16, stream: IO[str] = sys.stdin, device: str = "cuda") -> int:
+def run(model_dir: str, dtype: str, out_dir: str, max_tokens: int, block_size: int = 16, stream: IO[str] = sys.stdin, device: str = "cuda",
+        max_live: int = 8, enable_graphs: bool = False) -> int:
     os.makedirs(out_dir, exist_ok=True)
-    replayer = Replayer(model_dir, dtype, max_tokens, block_size=block_size, device=device)
+    replayer = Replayer(model_dir, dtype, max_tokens, block_size=block_size, device=device, max_live=max_live, enable_graphs=enable_graphs)
     for line in stream:
         line = line.strip()
         if not line:
