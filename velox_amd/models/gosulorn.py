@@ -173,8 +173,8 @@ def _recurrence_spec(config: GosulornConfig, sizes: Dict[str, Any], kind: str) -
         return PartSpec.of("linear_recurrence", rule="additive", decay="sigmoid_channel", gate="silu", unit_qk=False, tau=sizes["tau"],
                            decay_rank=sizes["ranks"]["a1"], **common)
     if kind == "delta":
-        return PartSpec.of("linear_recurrence", rule="delta", decay="head", gate="silu", unit_qk=True, **common)
-    return PartSpec.of("linear_recurrence", rule="delta", decay="channel", gate="sigmoid_low_rank", unit_qk=True,
+        return PartSpec.of("linear_recurrence", rule="delta", decay="head", gate="silu", unit_qk=True, qkv_silu=True, **common)
+    return PartSpec.of("linear_recurrence", rule="delta", decay="channel", gate="sigmoid_low_rank", unit_qk=True, qkv_silu=True,
                        decay_rank=sizes["ranks"]["a1"], gate_rank=sizes["ranks"]["g1"], **common)
 
 

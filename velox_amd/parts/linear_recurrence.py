@@ -11,7 +11,8 @@ per head, or one per head and key channel: it multiplies rows), a key ``k_t``, a
 * q and k have ``kv_heads`` heads of ``dim`` channels, v has ``heads`` heads of ``vdim``; head ``h`` reads q/k head
   ``h // (heads / kv_heads)``.  q is multiplied by ``dim ** -0.5``.
 * ``conv_taps``: q, k and v pass a short causal convolution per channel (``y_t = sum_j w[:, j] u_(t - taps + 1 + j)``, zeros
-  before the start) and then SiLU; the last ``taps - 1`` projected rows of a sequence are part of its state.
+  before the start) and then SiLU; the last ``taps - 1`` projected rows of a sequence are part of its state.  With
+  ``qkv_silu`` and no convolution the SiLU alone remains (a convolution of one tap whose weights are ones).
 * ``unit_qk``: q and k become unit vectors per head, ``x / sqrt(sum(x^2) + 1e-6)`` (before q's factor).
 * ``decay``:
   ``"head"``             ``g = exp(-exp(A_log_h) softplus(W_a x + dt_bias_h))``, one per head;
@@ -47,7 +48,7 @@ _DEFAULT_NAMES = {"q": "q", "k": "k", "v": "v", "o": "o", "beta": "b", "A_log": 
 
 class LinearRecurrenceMixer(Mixer):
     def __init__(self, prefix: str, hidden_size: int, num_heads: int, num_kv_heads: int, dim: int, vdim: int, norm_eps: float,
-                 rule: str = "delta", decay: str = "head", gate: str = "silu", conv_taps: int = 0, unit_qk: bool = False,
+                 rule: str = "delta", decay: str = "head", gate: str = "silu", conv_taps: int = 0, unit_qk: bool = False, qkv_silu: bool = False,
                  decay_rank: Optional[int] = None, gate_rank: Optional[int] = None, tau: float = 1.0,
                  names: Tuple[Tuple[str, str], ...] = ()) -> None:
         """``decay_rank`` / ``gate_rank``: the inner sizes of the low-rank maps (rows of ``a1`` / ``g1``)."""
@@ -75,6 +76,7 @@ class LinearRecurrenceMixer(Mixer):
         self.rule, self.decay, self.gate = rule, decay, gate
         self.conv_taps = int(conv_taps)
         self.unit_qk = bool(unit_qk)
+        self.qkv_silu = bool(qkv_silu)
         self.decay_rank = int(decay_rank or 0) if decay != "head" else 0
         self.gate_rank = int(gate_rank or 0) if gate == "sigmoid_low_rank" else 0
         self.tau = float(tau)
@@ -151,6 +153,8 @@ class LinearRecurrenceMixer(Mixer):
                 wide[at:, self.decay_rank:] = self.g2_weight
             self.low_out_weight = wide
         self._prepared.pop("low_out_weight", None)
+        if self.conv_taps == 0 and self.qkv_silu and self.main_weight is not None:
+            self.conv_weight = torch.ones((self.conv_channels, 1), dtype=torch.float32, device=self.main_weight.device)
         if self.decay == "sigmoid_channel":
             if self.a2_bias is not None:
                 self.decay_rate = torch.full((self.num_heads,), 1.0 / self.tau, dtype=torch.float32, device=self.a2_bias.device)
@@ -180,7 +184,7 @@ class LinearRecurrenceMixer(Mixer):
         heads, kv_heads, dim, vdim = self.num_heads, self.num_kv_heads, self.dim, self.vdim
         main = ops.linear(x, self.operand("main_weight"), None, ctx.dtype)
         qkv, q_at, k_at, v_at = main, 0, self.q_size, self.q_size + self.k_size
-        if self.conv_taps >= 1:
+        if self.conv_taps >= 1 or self.qkv_silu:
             tail = cache.tensors["conv_tail"] if self.conv_taps >= 2 else None
             qkv = ops.short_conv(main, self.conv_channels, self.conv_weight, tail, ctx.slots, ctx.cu_q, ctx.max_q_len, activation="silu")
         low = None
