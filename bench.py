@@ -16,7 +16,9 @@ over the steps in which all of them decode, ``..._frac``: that step's share of t
 ``e2e_b<B>_p512_g256``: generated tokens / wall time with the prompts' time included, which is how
 the reference's ``benchmark.py:204`` counts).
 
-``--design dipisun`` does for the Dipisun design what ``--design tiverax`` does for Tiverax, beside Tiverax with the same experts and
+``--design gosulorn`` measures the Gosulorn design (residual streams, attention over a sliding window beside a gated delta rule, gated
+linear attention, delta rules; every mixer's memory a state of fixed size or a window's pages) beside the dense decoder of the same width,
+depth, heads and feed-forward size; ``--design dipisun`` does for the Dipisun design what ``--design tiverax`` does for Tiverax, beside Tiverax with the same experts and
 the dense decoder with the same heads.  ``--design tiverax`` measures something else and leaves the above untouched: prefill and decode throughput of the Tiverax
 design (attention over a cached latent, routed experts) at layer sizes of real models, beside the Qwen2 dense decoder
 with the same width, depth, heads and dense feed-forward size, as one JSON line of its own.
@@ -275,6 +277,30 @@ def dipisun_config(size: dict) -> dict:
     return {"architecture": "Dipisun", "vocab": DESIGN_VOCAB, "width": size["width"], "norm": {"eps": 1e-5}, "residual_mult": 0.5, "layers": layers}
 
 
+# Layer sizes for --design gosulorn: eight layers, parallel (window attention beside a delta rule with a decay per key channel),
+# gated linear attention, parallel, delta rule, twice over; four residual streams; head sizes of 128 as the dense decoder beside it.
+GOSULORN_SIZES = {
+    "2k": dict(width=2048, streams=4, ff=5632, heads=16, kv_heads=4, dim=128, window=1024, right_heads=8, gla_heads=8, gla_vdim=256, delta_heads=16, delta_kv_heads=8, rank=64),
+    "4k": dict(width=4096, streams=4, ff=11008, heads=32, kv_heads=8, dim=128, window=2048, right_heads=16, gla_heads=16, gla_vdim=256, delta_heads=32, delta_kv_heads=16, rank=128),
+}
+
+
+def gosulorn_config(size: dict) -> dict:
+    dim = size["dim"]
+    left = {"heads": size["heads"], "kv_heads": size["kv_heads"], "dim": dim, "vdim": dim, "scale": dim ** -0.5, "conv": 4, "mask": {"size": size["window"]},
+            "rot": {"dims": dim // 2, "base": 1e6, "scaling": {"factor": 4.0}}}
+    right = {"heads": size["right_heads"], "kv_heads": size["right_heads"], "dim": dim, "vdim": dim, "conv": 4, "a1_rank": size["rank"], "g1_rank": size["rank"]}
+    kinds = {
+        "parallel": {"left": left, "right": right, "left_scale": 0.8, "right_scale": 1.1},
+        "gla": {"heads": size["gla_heads"], "dim": dim, "vdim": size["gla_vdim"], "tau": 16.0, "a1_rank": size["rank"]},
+        "delta": {"heads": size["delta_heads"], "kv_heads": size["delta_kv_heads"], "dim": dim, "vdim": dim, "conv": 4},
+    }
+    mlp = {"kind": "dense", "ff": size["ff"]}
+    order = ("parallel", "gla", "parallel", "delta")
+    layers = [{"type": order[index % 4], "mixer": kinds[order[index % 4]], "mlp": mlp} for index in range(DESIGN_LAYERS)]
+    return {"architecture": "Gosulorn", "vocab": DESIGN_VOCAB, "width": size["width"], "norm": {"eps": 1e-5}, "streams": size["streams"], "layers": layers}
+
+
 def tiverax_all_routed(size: dict) -> dict:
     """Tiverax at the width of ``size`` with the same experts per layer and per token (no shared expert, no dense layers)."""
     config = tiverax_config(dict(TIVERAX_SIZES["2k" if size["width"] == 2048 else "4k"], experts=size["experts"], top=size["top"], expert_ff=size["expert_ff"]))
@@ -288,6 +314,9 @@ def designs_at(design: str, name: str):
     if design == "tiverax":
         size = TIVERAX_SIZES[name]
         return (("tiverax", tiverax_config(size)), ("qwen2", qwen2_like(size)))
+    if design == "gosulorn":
+        size = GOSULORN_SIZES[name]
+        return (("gosulorn", gosulorn_config(size)), ("qwen2", qwen2_like(dict(size, rot_dim=0))))
     size = DIPISUN_SIZES[name]
     dense = dict(width=size["width"], heads=size["heads"], kv_heads=size["kv_heads"], dim=size["dim"], rot_dim=0, ff=size["top"] * size["expert_ff"])
     return (("dipisun", dipisun_config(size)), ("tiverax", tiverax_all_routed(size)), ("qwen2", qwen2_like(dense)))
@@ -311,7 +340,8 @@ def design_points(args) -> dict:
             parameters = sum(t.numel() for _, t in __import__("velox_amd.weights", fromlist=["named_tensors"]).named_tensors(engine.model))
             out[f"{label}_{name}"] = {"decode_tok_s": round(args.batch / step_s, 1), "decode_ms": round(step_s * 1000, 3), "decode_b1_ms": round(one_s * 1000, 3),
                                       "prefill_tok_s": round(args.prefill_tokens / prefill_s, 1), "prefill_ms": round(prefill_s * 1000, 3),
-                                      "parameters_m": round(parameters / 1e6, 1), "cache_bytes_per_token": engine.cache.bytes_per_page() // 16}
+                                      "parameters_m": round(parameters / 1e6, 1), "cache_bytes_per_token": engine.cache.bytes_per_page() // 16,
+                                      "state_bytes_per_request": sum(t[0].numel() * t.element_size() for group in engine.cache.state.tensors.values() for t in group.values())}
             engine.abort_all()
             del engine
             gc.collect()
@@ -336,7 +366,7 @@ def main() -> int:
     parser.add_argument("--shape", default="7b", choices=sorted(SHAPES), help="layer sizes: the headline is 7b; 1.5b and 32b are the reference's other two")
     parser.add_argument("--far", action="store_true",
                         help="further sizes under `points`: decode at batch 1 and 8 behind 32,256 tokens, a prefill of 8,192 tokens, and a decode step of a true float32 run (batch 8)")
-    parser.add_argument("--design", default=None, choices=["tiverax", "dipisun"],
+    parser.add_argument("--design", default=None, choices=["tiverax", "dipisun", "gosulorn"],
                         help="instead of the headline: prefill and decode of this design at real layer sizes beside the framework's closest models of equal size")
     parser.add_argument("--only", default="", help="with --design: which of the models that are measured side by side (names with commas between them; default: all)")
     parser.add_argument("--sizes", default="2k,4k", help="with --design: which of the sizes (2k, 4k = the models' widths)")
@@ -350,7 +380,7 @@ def main() -> int:
         points = design_points(args)
         first = args.sizes.split(",")[0]
         head = points.get(f"{args.design}_{first}") or next(iter(points.values()))
-        sizes = TIVERAX_SIZES if args.design == "tiverax" else DIPISUN_SIZES
+        sizes = {"tiverax": TIVERAX_SIZES, "dipisun": DIPISUN_SIZES, "gosulorn": GOSULORN_SIZES}[args.design]
         print(json.dumps({
             "metric": "decode_tokens_per_second", "value": head["decode_tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": args.steps,
             "warmup": args.warmup, "ms_per_step": head["decode_ms"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
