@@ -4,7 +4,7 @@
 //   short_conv          causal convolution over a few taps per channel, the inputs before a portion's start from the state slot
 //   rotate_pad_write    partial rotation of q and k, q at the attention kernels' head size, k and v into the paged cache
 //   recurrence_prepare  unit q and k, decay and beta of a linear recurrence, all float32
-//   linear_scan         the recurrence itself, token by token from the state slot
+//   linear_scan         the recurrence itself, token by token from the state slot (portions of prompts staged through LDS)
 //   gated_head_norm     RMS norm of each head's read-out, a shared weight, a gate
 // Everything between a load and a store is float32; stores round once.  No result depends on how a sequence's tokens
 // were cut into steps or on what else is in the batch: sums run in an order that only the sizes fix.
@@ -389,8 +389,16 @@ extern "C" int velox_recurrence_prepare(const void* qkv, int qkv_dtype, int ld, 
 // Every column of S is a recurrence of its own:   s <- g * s;  u = beta (v_e - k . s)  (delta rule)  or  u = v_e;
 // s <- s + k u;  o_e = q . s.   A column is held by R lanes of a wave, SCAN_ROWS consecutive rows each (R the smallest power of
 // two with R * SCAN_ROWS >= dim: a function of dim alone, so the order of every sum is too); the two dot products are
-// reduced over those lanes.  The next token's q, k, decay, value and beta are loaded while the current one is worked on.
+// summed in four interleaved parts per lane and then over those lanes (scan_token, the one place where a token is worked).
 // Grid (column blocks, heads, sequences); a workgroup of 256 lanes holds 256 / R columns.
+//   linear_scan_kernel         steps of single tokens: a token's q, k, decay, value and beta come straight from memory, the
+//                              next token's while the current one is worked on.
+//   linear_scan_staged_kernel  portions of prompts: the tokens are a dependent chain, so a token must cost no memory round
+//                              trip.  The workgroup carries the next block of tokens (q, k, decay of the head, the values of its
+//                              columns, beta) from memory into registers before it works through the current block out of
+//                              LDS, and writes the registers to the other LDS buffer behind it: one barrier per block, the
+//                              loads' latency lies behind a block's arithmetic.
+// Both give the same bits: they differ in where the operands wait, not in what is done with them.
 // ---------------------------------------------------------------------------------------------
 #define SCAN_ROWS 16
 
@@ -419,6 +427,35 @@ __device__ __forceinline__ void scan_load_rows(const float* __restrict__ p, int 
 #pragma unroll
     for (int i = 0; i < SCAN_ROWS; ++i) r[i] = d0 + i < dim ? p[d0 + i] : fill;
   }
+}
+
+// One token of one column: returns the read-out (complete in every lane of the column).
+template <int R>
+__device__ __forceinline__ float scan_token(float (&s)[SCAN_ROWS], const float (&q)[SCAN_ROWS], const float (&k)[SCAN_ROWS], const float (&dec)[SCAN_ROWS],
+                                            float val, float bet, int delta) {
+  float d[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int i = 0; i < SCAN_ROWS; ++i) {
+    s[i] *= dec[i];
+    d[i & 3] += s[i] * k[i];
+  }
+  float u = val;
+  if (delta) {
+    float dot = (d[0] + d[1]) + (d[2] + d[3]);
+#pragma unroll
+    for (int off = 1; off < R; off <<= 1) dot += __shfl_xor(dot, off, VELOX_WAVE);
+    u = bet * (val - dot);
+  }
+  float p[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int i = 0; i < SCAN_ROWS; ++i) {
+    s[i] += k[i] * u;
+    p[i & 3] += s[i] * q[i];
+  }
+  float o = (p[0] + p[1]) + (p[2] + p[3]);
+#pragma unroll
+  for (int off = 1; off < R; off <<= 1) o += __shfl_xor(o, off, VELOX_WAVE);
+  return o;
 }
 
 template <int R>
@@ -458,30 +495,156 @@ __global__ void __launch_bounds__(256) linear_scan_kernel(const ScanArgs a) {
   fetch(lo, q, k, dec, val, bet);
   for (int t = lo; t < hi; ++t) {
     if (t + 1 < hi) fetch(t + 1, qn, kn, decn, valn, betn);
-    float dot = 0.f;
-#pragma unroll
-    for (int i = 0; i < SCAN_ROWS; ++i) {
-      s[i] *= dec[i];
-      dot += s[i] * k[i];
-    }
-    float u = val;
-    if (a.delta) {
-#pragma unroll
-      for (int off = 1; off < R; off <<= 1) dot += __shfl_xor(dot, off, VELOX_WAVE);
-      u = bet * (val - dot);
-    }
-    float o = 0.f;
-#pragma unroll
-    for (int i = 0; i < SCAN_ROWS; ++i) {
-      s[i] += k[i] * u;
-      o += s[i] * q[i];
-    }
-#pragma unroll
-    for (int off = 1; off < R; off <<= 1) o += __shfl_xor(o, off, VELOX_WAVE);
+    const float o = scan_token<R>(s, q, k, dec, val, bet, a.delta);
     if (live && r == 0) a.out[((size_t)t * a.heads + h) * vdim + e] = o;
 #pragma unroll
     for (int i = 0; i < SCAN_ROWS; ++i) { q[i] = qn[i]; k[i] = kn[i]; dec[i] = decn[i]; }
     val = valn; bet = betn;
+  }
+  if (live) {
+#pragma unroll
+    for (int i = 0; i < SCAN_ROWS; ++i)
+      if (d0 + i < dim) S[(size_t)(d0 + i) * vdim] = s[i];
+  }
+}
+
+// A token's place in a staging buffer, in floats: q [dim], k [dim], the decay per channel [dim] if there is one, the values of
+// the workgroup's columns [256 / R], then beta and the head's decay (and two floats that keep the next token 16-byte aligned).
+#define STAGE_PIECES 8  // 16-byte pieces of q, k and decay that one lane carries per block of tokens, at most
+#define STAGE_VALUES 4  // values that one lane carries per block, at most
+
+template <int R>
+__global__ void __launch_bounds__(256) linear_scan_staged_kernel(const ScanArgs a, const int block_tokens) {
+  extern __shared__ float4_t stage_pieces[];
+  float* stage = reinterpret_cast<float*>(stage_pieces);
+  constexpr int COLS = 256 / R;
+  const int tid = threadIdx.x;
+  const int r = tid % R, c_local = tid / R;
+  const int e = blockIdx.x * COLS + c_local;
+  const int h = blockIdx.y, b = blockIdx.z;
+  const int lo = a.cu_q[b], hi = a.cu_q[b + 1];
+  if (hi <= lo) return;  // (the whole workgroup: no barrier is left waiting)
+  const bool live = e < a.vdim;
+  const int col = live ? e : a.vdim - 1;
+  const int dim = a.dim, vdim = a.vdim, heads = a.heads;
+  const int d0 = r * SCAN_ROWS;
+  const int g = h / (heads / a.kv_heads);
+  const int per_channel = a.decay_per_channel;
+  const int qk_pieces = dim / 2;                                     // (2 * dim floats in pieces of 4)
+  const int pieces_per_token = qk_pieces + (per_channel ? dim / 4 : 0);
+  const int values_at = 2 * dim + (per_channel ? dim : 0);
+  const int scalars_at = values_at + COLS;
+  const int stride = scalars_at + 4;
+
+  // what this lane carries from memory to LDS in every block: token within the block, offset within the token's row, place in LDS
+  int piece_token[STAGE_PIECES], piece_from[STAGE_PIECES], piece_to[STAGE_PIECES];
+#pragma unroll
+  for (int p = 0; p < STAGE_PIECES; ++p) {
+    const int index = tid + p * 256;
+    const int token = index / pieces_per_token, piece = index - token * pieces_per_token;
+    piece_token[p] = token < block_tokens ? token : -1;
+    piece_from[p] = piece < qk_pieces ? piece * 4 : -1 - (piece - qk_pieces) * 4;  // (negative: a piece of the decay)
+    piece_to[p] = token * stride + piece * 4;
+  }
+  float4_t carried[STAGE_PIECES];
+  float carried_values[STAGE_VALUES];
+  float carried_beta = 1.f, carried_decay = 1.f;
+  auto load_block = [&](int t0) {
+#pragma unroll
+    for (int p = 0; p < STAGE_PIECES; ++p) {
+      const int t = t0 + piece_token[p];
+      if (piece_token[p] >= 0 && t < hi) {
+        const float* from = piece_from[p] >= 0 ? a.qk + ((size_t)t * a.kv_heads + g) * 2 * dim + piece_from[p]
+                                               : a.decay + ((size_t)t * heads + h) * dim + (-1 - piece_from[p]);
+        carried[p] = *reinterpret_cast<const float4_t*>(from);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < STAGE_VALUES; ++j) {
+      const int index = tid + j * 256;
+      const int token = index / COLS, c = index % COLS;
+      const int t = t0 + token, column = blockIdx.x * COLS + c;
+      if (token < block_tokens && t < hi)
+        carried_values[j] = column < vdim ? load_as_f32(a.v, a.v_bf16, (size_t)t * a.v_ld + a.v_at + (size_t)h * vdim + column) : 0.f;
+    }
+    if (tid < block_tokens && t0 + tid < hi) {
+      carried_beta = a.beta ? a.beta[(size_t)(t0 + tid) * heads + h] : 1.f;
+      carried_decay = per_channel ? 1.f : a.decay[(size_t)(t0 + tid) * heads + h];
+    }
+  };
+  auto store_block = [&](int buffer) {  // (rows of tokens beyond the sequence's end keep what they held: nobody reads them)
+    const int at = buffer * block_tokens * stride;
+#pragma unroll
+    for (int p = 0; p < STAGE_PIECES; ++p)
+      if (piece_token[p] >= 0) *reinterpret_cast<float4_t*>(&stage[at + piece_to[p]]) = carried[p];
+#pragma unroll
+    for (int j = 0; j < STAGE_VALUES; ++j) {
+      const int index = tid + j * 256;
+      const int token = index / COLS, c = index % COLS;
+      if (token < block_tokens) stage[at + token * stride + values_at + c] = carried_values[j];
+    }
+    if (tid < block_tokens) {
+      stage[at + tid * stride + scalars_at] = carried_beta;
+      stage[at + tid * stride + scalars_at + 1] = carried_decay;
+    }
+  };
+#pragma unroll
+  for (int p = 0; p < STAGE_PIECES; ++p) carried[p] = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int j = 0; j < STAGE_VALUES; ++j) carried_values[j] = 0.f;
+
+  float* S = a.state + (((size_t)a.slots[b] * heads + h) * dim) * vdim + col;
+  float s[SCAN_ROWS];
+#pragma unroll
+  for (int i = 0; i < SCAN_ROWS; ++i) s[i] = d0 + i < dim ? S[(size_t)(d0 + i) * vdim] : 0.f;
+
+  float q[SCAN_ROWS], k[SCAN_ROWS], dec[SCAN_ROWS], qn[SCAN_ROWS], kn[SCAN_ROWS], decn[SCAN_ROWS];
+  float val, bet, valn = 0.f, betn = 1.f;
+  auto fetch = [&](int at, float (&fq)[SCAN_ROWS], float (&fk)[SCAN_ROWS], float (&fd)[SCAN_ROWS], float& fv, float& fb) {
+    const float one = stage[at + scalars_at + 1];
+#pragma unroll
+    for (int i = 0; i < SCAN_ROWS; i += 4) {
+      if (d0 + i < dim) {  // (dim is a multiple of 4 here: a piece lies inside the head or outside)
+        const float4_t x = *reinterpret_cast<const float4_t*>(&stage[at + d0 + i]);
+        const float4_t y = *reinterpret_cast<const float4_t*>(&stage[at + dim + d0 + i]);
+        fq[i] = x[0]; fq[i + 1] = x[1]; fq[i + 2] = x[2]; fq[i + 3] = x[3];
+        fk[i] = y[0]; fk[i + 1] = y[1]; fk[i + 2] = y[2]; fk[i + 3] = y[3];
+        if (per_channel) {
+          const float4_t z = *reinterpret_cast<const float4_t*>(&stage[at + 2 * dim + d0 + i]);
+          fd[i] = z[0]; fd[i + 1] = z[1]; fd[i + 2] = z[2]; fd[i + 3] = z[3];
+        } else {
+          fd[i] = fd[i + 1] = fd[i + 2] = fd[i + 3] = one;
+        }
+      } else {
+        fq[i] = fq[i + 1] = fq[i + 2] = fq[i + 3] = 0.f;
+        fk[i] = fk[i + 1] = fk[i + 2] = fk[i + 3] = 0.f;
+        fd[i] = fd[i + 1] = fd[i + 2] = fd[i + 3] = 1.f;
+      }
+    }
+    fv = stage[at + values_at + c_local];
+    fb = stage[at + scalars_at];
+  };
+
+  load_block(lo);
+  store_block(0);
+  __syncthreads();
+  int buffer = 0;
+  for (int t0 = lo; t0 < hi; t0 += block_tokens, buffer ^= 1) {
+    const bool more = t0 + block_tokens < hi;
+    if (more) load_block(t0 + block_tokens);
+    const int count = hi - t0 < block_tokens ? hi - t0 : block_tokens;
+    const int at = buffer * block_tokens * stride;
+    fetch(at, q, k, dec, val, bet);
+    for (int j = 0; j < count; ++j) {
+      if (j + 1 < count) fetch(at + (j + 1) * stride, qn, kn, decn, valn, betn);
+      const float o = scan_token<R>(s, q, k, dec, val, bet, a.delta);
+      if (live && r == 0) a.out[((size_t)(t0 + j) * heads + h) * vdim + e] = o;
+#pragma unroll
+      for (int i = 0; i < SCAN_ROWS; ++i) { q[i] = qn[i]; k[i] = kn[i]; dec[i] = decn[i]; }
+      val = valn; bet = betn;
+    }
+    if (more) store_block(buffer ^ 1);  // (the buffer that the block before this one was worked from: everyone is past the barrier behind it)
+    __syncthreads();
   }
   if (live) {
 #pragma unroll
@@ -496,15 +659,42 @@ extern "C" int velox_linear_scan_lanes(int dim) {
   return lanes;
 }
 
+// Tokens per staging block: as many as the lanes can carry and two buffers of LDS can hold, 16 at most; 0: no staging.
+static int scan_block_tokens(int dim, int lanes, int per_channel) {
+  if (dim % 4 != 0) return 0;
+  const int cols = 256 / lanes;
+  const int pieces = dim / 2 + (per_channel ? dim / 4 : 0);
+  const int stride = 2 * dim + (per_channel ? dim : 0) + cols + 4;
+  int tokens = 16;
+  while (tokens >= 2 && (tokens * pieces > 256 * STAGE_PIECES || tokens * cols > 256 * STAGE_VALUES || 2 * tokens * stride * (int)sizeof(float) > 60 * 1024))
+    tokens >>= 1;
+  return tokens >= 2 ? tokens : 0;
+}
+
 extern "C" int velox_linear_scan(const float* qk, const void* v, int v_dtype, int v_ld, int v_at, const float* decay, int decay_per_channel, const float* beta,
-                                 float* state, const int* slots, const int* cu_q, float* out, int num_seqs, int heads, int kv_heads, int dim, int vdim,
-                                 int delta, hipStream_t stream) {
+                                 float* state, const int* slots, const int* cu_q, float* out, int num_seqs, int max_q_len, int heads, int kv_heads, int dim,
+                                 int vdim, int delta, hipStream_t stream) {
   if (num_seqs <= 0) return 0;
   const int lanes = velox_linear_scan_lanes(dim);
   if (lanes > 64 || heads > 65535 || num_seqs > 65535 || kv_heads < 1 || heads % kv_heads != 0 || (delta && !beta)) return (int)hipErrorInvalidValue;
   ScanArgs a{qk, v, v_dtype == VELOX_BF16, v_ld, v_at, decay, decay_per_channel, beta, state, slots, cu_q, out, heads, kv_heads, dim, vdim, delta};
   const int cols = 256 / lanes;
   const dim3 grid((vdim + cols - 1) / cols, heads, num_seqs);
+  const int block_tokens = max_q_len > 2 ? scan_block_tokens(dim, lanes, decay_per_channel) : 0;
+  if (block_tokens > 0) {
+    const int stride = 2 * dim + (decay_per_channel ? dim : 0) + cols + 4;
+    const size_t lds = (size_t)2 * block_tokens * stride * sizeof(float);
+    switch (lanes) {
+      case 1: linear_scan_staged_kernel<1><<<grid, 256, lds, stream>>>(a, block_tokens); break;
+      case 2: linear_scan_staged_kernel<2><<<grid, 256, lds, stream>>>(a, block_tokens); break;
+      case 4: linear_scan_staged_kernel<4><<<grid, 256, lds, stream>>>(a, block_tokens); break;
+      case 8: linear_scan_staged_kernel<8><<<grid, 256, lds, stream>>>(a, block_tokens); break;
+      case 16: linear_scan_staged_kernel<16><<<grid, 256, lds, stream>>>(a, block_tokens); break;
+      case 32: linear_scan_staged_kernel<32><<<grid, 256, lds, stream>>>(a, block_tokens); break;
+      default: linear_scan_staged_kernel<64><<<grid, 256, lds, stream>>>(a, block_tokens); break;
+    }
+    VELOX_RETURN_LAUNCH_STATUS();
+  }
   switch (lanes) {
     case 1: linear_scan_kernel<1><<<grid, 256, 0, stream>>>(a); break;
     case 2: linear_scan_kernel<2><<<grid, 256, 0, stream>>>(a); break;

@@ -100,6 +100,7 @@ class HipOps:
         self.fuse_residual_norm = True
         self.use_grouped_mfma = True  # (False: the grouped bfloat16 products take the exact multiply-add tiles, for tests)
         self._mm_out_dtype_ok: Optional[bool] = None
+        self._bias_copies: Dict[Tuple[int, int], Tuple[torch.Tensor, torch.Tensor]] = {}
         self._raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
 
     # -- loading --------------------------------------------------------------------------------
@@ -164,7 +165,7 @@ class HipOps:
         c.velox_short_conv.argtypes = [_P, _I, _I, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P]
         c.velox_rotate_pad_write.argtypes = [_P, _I, _P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P]
         c.velox_recurrence_prepare.argtypes = [_P, _I, _I, _I, _I, _I, _I, _I, _F, _P, _I, _I, _I, _I, _I, _P, _P, _F, _P, _I, _I, _I, _P, _P, _P, _I, _P]
-        c.velox_linear_scan.argtypes = [_P, _P, _I, _I, _I, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P]
+        c.velox_linear_scan.argtypes = [_P, _P, _I, _I, _I, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]
         c.velox_linear_scan_lanes.argtypes = [_I]
         c.velox_gated_head_norm.argtypes = [_P, _P, _F, _P, _I, _I, _I, _I, _P, _I, _I, _I, _I, _P]
         for fn in (c.velox_stream_norm, c.velox_embed_copies, c.velox_gated_act_mul, c.velox_short_conv, c.velox_rotate_pad_write, c.velox_recurrence_prepare,
@@ -548,6 +549,9 @@ class HipOps:
         skinny_rows = 16 if n > 8192 else 32  # measured on MI355X: beyond this the library's kernels stream faster
         if self.use_skinny_gemm and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and m <= skinny_rows and k % 64 == 0:
             return self.skinny_gemm(x, weight, bias, out_dtype, packed=packed, x_packed=self._packed_rows_of(x, k))
+        if self.use_library_gemm and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and bias is not None and out_dtype == torch.bfloat16:
+            # the library adds a bias of the product's own dtype to its float32 sums before the one rounding
+            return torch.nn.functional.linear(x, weight, self._bias_in_bfloat16(bias))
         if self.use_library_gemm and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and bias is None:
             if out_dtype == torch.bfloat16:
                 return torch.nn.functional.linear(x, weight)
@@ -556,6 +560,16 @@ class HipOps:
                     self._decide_float32_out_route()
                 return torch.mm(x, weight.t(), out_dtype=torch.float32)
         return self.gemm_fma(x, weight, bias, out_dtype)
+
+    def _bias_in_bfloat16(self, bias: torch.Tensor) -> torch.Tensor:
+        """A bfloat16 copy of a float32 bias vector, made once per vector (keyed by its storage; the float32 vector is kept
+        alive beside it, so the key cannot come to mean another tensor)."""
+        key = (bias.data_ptr(), bias.numel())
+        held = self._bias_copies.get(key)
+        if held is None or held[0] is not bias:
+            held = (bias, bias.to(torch.bfloat16))
+            self._bias_copies[key] = held
+        return held[1]
 
     def _decide_float32_out_route(self) -> None:
         """Decides once how a bfloat16 product with a float32 result and more rows than the skinny kernels take (the
@@ -930,7 +944,7 @@ class HipOps:
         self.linear_scan_supports(dim, vdim)
         out = torch.empty((tokens, heads * vdim), dtype=torch.float32, device=self.device)
         status = self._core.velox_linear_scan(_ptr(qk), _ptr(v_source), _code(v_source.dtype), v_source.shape[1], int(v_at), _ptr(decay), int(per_channel),
-                                              _ptr(beta) if delta else _P(0), _ptr(state), _ptr(slots), _ptr(cu_q), _ptr(out), slots.shape[0], int(heads),
+                                              _ptr(beta) if delta else _P(0), _ptr(state), _ptr(slots), _ptr(cu_q), _ptr(out), slots.shape[0], int(max_q_len), int(heads),
                                               int(kv_heads), int(dim), int(vdim), int(bool(delta)), self._stream())
         self._launched(status, "linear_scan")
         return out
