@@ -80,7 +80,7 @@ CONFIG_B = {
     ],
 }
 # Sizes the kernels for decode-sized bfloat16 batches and the matrix cores take (multiples of 64 and 8), key heads of 128
-# channels (a column of the state then spreads over eight lanes), two streams.
+# channels (a column of the state then spreads over sixteen lanes), two streams.
 _C0 = parallel(attention(4, 2, 64, 32, 0.2, window=24, conv=4, rot=(32, 10000.0, 4.0)), delta(4, 4, 32, 64, conv=3, rank=16, gate_rank=8), 0.9, 1.2)
 CONFIG_C = {
     "architecture": "Gosulorn", "vocab": 160, "width": 128, "norm": {"eps": 1e-5}, "streams": 2,

@@ -221,7 +221,8 @@ def test_recurrence_prepare_scan_and_head_norm(ops, ref, dtype, heads, kv_heads,
         near(ops.gated_head_norm(b, weight, 1e-6, low, cols, kind, heads, vdim, dt), ref.gated_head_norm(b, weight, 1e-6, low, cols, kind, heads, vdim, dt), REL[dtype], kind)
 
 
-@pytest.mark.parametrize("heads,kv_heads,dim,vdim,per_channel,delta_rule", [(4, 2, 64, 64, True, True), (2, 2, 128, 128, False, True), (3, 3, 32, 48, True, False)])
+@pytest.mark.parametrize("heads,kv_heads,dim,vdim,per_channel,delta_rule", [(4, 2, 64, 64, True, True), (2, 2, 128, 128, False, True), (3, 3, 32, 48, True, False), (2, 1, 256, 20, True, True),
+                                                                            (1, 1, 128, 9, True, False), (2, 2, 72, 40, False, True)])
 def test_a_long_portion_equals_its_pieces_and_its_first_token_is_kept(ops, ref, heads, kv_heads, dim, vdim, per_channel, delta_rule):
     """600 tokens in one step, in pieces (one of a single token, one of two) and against the plain loop; with decays
     close to 1 the first token's write still decides the last read-out."""
@@ -247,13 +248,19 @@ def test_a_long_portion_equals_its_pieces_and_its_first_token_is_kept(ops, ref, 
 
     whole, state = run(ops, (n,), values)
     pieces, state_pieces = run(ops, (1, 2, 300, 17, 280), values)
-    assert torch.equal(whole, pieces) and torch.equal(state, state_pieces)  # the order of every sum is fixed by the sizes alone
+    if dim % 64 == 0:  # (long portions of such heads run a kernel of their own, which sums in another order than single tokens do)
+        near(pieces, whole, 1e-5, "pieces")
+        near(state_pieces, state, 1e-5, "state of the pieces")
+        again, state_again = run(ops, (n,), values)
+        assert torch.equal(whole, again) and torch.equal(state, state_again)
+    else:  # the order of every sum is fixed by the sizes alone
+        assert torch.equal(whole, pieces) and torch.equal(state, state_pieces)
     want, want_state = run(ref, (n,), values)
     near(whole, want, 5e-5, "read-out")
     near(state, want_state, 5e-5, "state")
     without = values.clone()
     without[0] = 0.0
-    assert float((run(ref, (n,), without)[0][-1] - want[-1]).abs().max()) > 0.05 * float(want[-1].abs().max())
+    assert float((run(ref, (n,), without)[0][-50:] - want[-50:]).abs().max()) > 0.05 * float(want[-50:].abs().max())
 
 
 # ----------------------------------------------------------------------------------------------------

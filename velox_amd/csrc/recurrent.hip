@@ -106,6 +106,102 @@ __global__ void __launch_bounds__(256) stream_norm_kernel(const StreamNormArgs a
     store_from_f32(a.out, a.out_bf16, (size_t)row * H + i, (u_row[i] - mean) * inv * a.weight[i]);
 }
 
+// The same for rows of a multiple of four floats: a lane owns pieces of four neighbours (16-byte loads and stores of the
+// streams, 8-byte ones of bfloat16 terms and results), a workgroup is as wide as a row has pieces (1024 lanes at most), and
+// u stays in registers between the passes: PIECES pieces per lane, which the launch picks from the row's length.
+__device__ __forceinline__ float4_t load4_as_f32(const void* p, int is_bf16, size_t i) {
+  if (!is_bf16) return *reinterpret_cast<const float4_t*>((const float*)p + i);
+  const short4_t raw = *reinterpret_cast<const short4_t*>((const bf16_t*)p + i);
+  float4_t out;
+#pragma unroll
+  for (int c = 0; c < 4; ++c) out[c] = __uint_as_float(((unsigned)(unsigned short)raw[c]) << 16);
+  return out;
+}
+__device__ __forceinline__ void store4_from_f32(void* p, int is_bf16, size_t i, float4_t v) {
+  if (!is_bf16) { *reinterpret_cast<float4_t*>((float*)p + i) = v; return; }
+  short4_t raw;
+#pragma unroll
+  for (int c = 0; c < 4; ++c) raw[c] = bf16_bits(v[c]);
+  *reinterpret_cast<short4_t*>((bf16_t*)p + i) = raw;
+}
+
+template <int PIECES>
+__global__ void __launch_bounds__(1024) stream_norm_vec_kernel(const StreamNormArgs a) {
+  __shared__ float scratch[16];
+  __shared__ float coef[STREAMS_MAX * STREAMS_MAX + 2 * STREAMS_MAX];
+  const int S = a.streams, H = a.hidden, pieces = H / 4;
+  float* mix = coef;
+  float* ow = coef + STREAMS_MAX * STREAMS_MAX;
+  float* iw = ow + STREAMS_MAX;
+  if (threadIdx.x < S * S) {
+    const int s = threadIdx.x / S, t = threadIdx.x % S;
+    mix[s * STREAMS_MAX + t] = a.mix ? a.mix[s * S + t] : (s == t ? 1.f : 0.f);
+  }
+  if (threadIdx.x < S) {
+    ow[threadIdx.x] = a.out_w ? a.out_w[threadIdx.x] : 1.f;
+    iw[threadIdx.x] = a.in_w ? a.in_w[threadIdx.x] : 1.f;
+  }
+  __syncthreads();
+  const int row = blockIdx.x;
+  const size_t src = a.rows ? (size_t)a.rows[row] : (size_t)row;
+  float* res = a.residual + src * (size_t)S * H;
+  const bool update = a.num_terms > 0;
+  const bool write_back = update && a.rows == nullptr;
+  float4_t u[PIECES];
+  float sum = 0.f;
+#pragma unroll
+  for (int p = 0; p < PIECES; ++p) {
+    const int piece = threadIdx.x + p * blockDim.x;
+    u[p] = float4_t{0.f, 0.f, 0.f, 0.f};
+    if (piece >= pieces) continue;
+    const int i = piece * 4;
+    float4_t x[STREAMS_MAX];
+#pragma unroll
+    for (int s = 0; s < STREAMS_MAX; ++s)
+      if (s < S) x[s] = *reinterpret_cast<const float4_t*>(res + (size_t)s * H + i);
+    if (update) {
+      float4_t y = a.scale0 * load4_as_f32(a.term0, a.term0_bf16, src * H + i);
+      if (a.num_terms > 1) y += a.scale1 * load4_as_f32(a.term1, a.term1_bf16, src * H + i);
+#pragma unroll
+      for (int t = 0; t < STREAMS_MAX; ++t) {
+        if (t < S) {
+          float4_t n = float4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int s = 0; s < STREAMS_MAX; ++s)
+            if (s < S) n += mix[s * STREAMS_MAX + t] * x[s];
+          n += ow[t] * y;
+          if (write_back) *reinterpret_cast<float4_t*>(res + (size_t)t * H + i) = n;
+          u[p] += iw[t] * n;
+        }
+      }
+    } else {
+#pragma unroll
+      for (int s = 0; s < STREAMS_MAX; ++s)
+        if (s < S) u[p] += iw[s] * x[s];
+    }
+    sum += (u[p][0] + u[p][1]) + (u[p][2] + u[p][3]);
+  }
+  float mean = 0.f;
+  if (a.center) mean = block_sum(sum, scratch) / (float)H;
+  float sq = 0.f;
+#pragma unroll
+  for (int p = 0; p < PIECES; ++p) {
+    if (threadIdx.x + p * blockDim.x < pieces) {
+      const float4_t d = u[p] - mean;
+      sq += (d[0] * d[0] + d[1] * d[1]) + (d[2] * d[2] + d[3] * d[3]);
+    }
+  }
+  const float inv = 1.f / sqrtf(block_sum(sq, scratch) / (float)H + a.eps);
+#pragma unroll
+  for (int p = 0; p < PIECES; ++p) {
+    const int piece = threadIdx.x + p * blockDim.x;
+    if (piece < pieces) {
+      const float4_t w = *reinterpret_cast<const float4_t*>(a.weight + piece * 4);
+      store4_from_f32(a.out, a.out_bf16, (size_t)row * H + piece * 4, (u[p] - mean) * inv * w);
+    }
+  }
+}
+
 extern "C" int velox_stream_norm(float* residual, const void* term0, int term0_dtype, float scale0, const void* term1, int term1_dtype, float scale1,
                                  int num_terms, const float* mix, const float* out_w, const float* in_w, const float* weight, const int* rows,
                                  void* out, int out_dtype, int count, int hidden, int streams, int center, float eps, hipStream_t stream) {
@@ -113,6 +209,17 @@ extern "C" int velox_stream_norm(float* residual, const void* term0, int term0_d
   if (streams < 1 || streams > STREAMS_MAX || hidden < 1 || hidden > 16384 || num_terms < 0 || num_terms > 2) return (int)hipErrorInvalidValue;
   StreamNormArgs a{residual, term0, term1, term0_dtype == VELOX_BF16, term1_dtype == VELOX_BF16, num_terms, scale0, scale1, mix, out_w, in_w, weight,
                    rows, out, out_dtype == VELOX_BF16, hidden, streams, center, eps};
+  const uintptr_t addresses = (uintptr_t)residual | (uintptr_t)weight | (uintptr_t)out | (uintptr_t)term0 | (uintptr_t)term1;
+  if (hidden % 4 == 0 && addresses % 16 == 0) {  // (rows are a multiple of four elements, so their pieces are as aligned as the tensors)
+    const int pieces = hidden / 4;
+    int lanes = (pieces + 63) / 64 * 64;
+    if (lanes > 1024) lanes = 1024;
+    const int per_lane = (pieces + lanes - 1) / lanes;
+    if (per_lane == 1) stream_norm_vec_kernel<1><<<count, lanes, 0, stream>>>(a);
+    else if (per_lane == 2) stream_norm_vec_kernel<2><<<count, lanes, 0, stream>>>(a);
+    else stream_norm_vec_kernel<4><<<count, lanes, 0, stream>>>(a);
+    VELOX_RETURN_LAUNCH_STATUS();
+  }
   stream_norm_kernel<<<count, 256, (size_t)hidden * sizeof(float), stream>>>(a);
   VELOX_RETURN_LAUNCH_STATUS();
 }
@@ -390,6 +497,7 @@ extern "C" int velox_recurrence_prepare(const void* qkv, int qkv_dtype, int ld, 
 // s <- s + k u;  o_e = q . s.   A column is held by R lanes of a wave, SCAN_ROWS consecutive rows each (R the smallest power of
 // two with R * SCAN_ROWS >= dim: a function of dim alone, so the order of every sum is too); the two dot products are
 // summed in four interleaved parts per lane and then over those lanes (scan_token, the one place where a token is worked).
+// With eight rows to a lane a head of 128 key channels spreads over sixteen lanes, and a workgroup holds sixteen columns.
 // Grid (column blocks, heads, sequences); a workgroup of 256 lanes holds 256 / R columns.
 //   linear_scan_kernel         steps of single tokens: a token's q, k, decay, value and beta come straight from memory, the
 //                              next token's while the current one is worked on.
@@ -398,9 +506,29 @@ extern "C" int velox_recurrence_prepare(const void* qkv, int qkv_dtype, int ld, 
 //                              columns, beta) from memory into registers before it works through the current block out of
 //                              LDS, and writes the registers to the other LDS buffer behind it: one barrier per block, the
 //                              loads' latency lies behind a block's arithmetic.
-// Both give the same bits: they differ in where the operands wait, not in what is done with them.
+//   linear_scan_wave_kernel    the same for dim = 64, 128, 256, 512, a column per wave (described at the kernel).
+// The first two give the same bits: they differ in where the operands wait, not in what is done with them; the third sums in
+// another order (which, like theirs, only the sizes fix).
 // ---------------------------------------------------------------------------------------------
-#define SCAN_ROWS 16
+#define SCAN_ROWS 8
+
+// Sum over the R lanes that hold a column (R a power of two, the lanes consecutive and aligned): pairs, quads, halves of a
+// row of 16 and the row by data-parallel moves inside the vector unit, beyond a row through the cross-lane network.  Both
+// partners of a step add the same two numbers, so every lane ends with the same bits.
+template <int CTRL>
+__device__ __forceinline__ float lanes_moved(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
+}
+template <int R>
+__device__ __forceinline__ float sum_over_lanes(float v) {
+  if (R >= 2) v += lanes_moved<0xB1>(v);    // quad_perm [1, 0, 3, 2]
+  if (R >= 4) v += lanes_moved<0x4E>(v);    // quad_perm [2, 3, 0, 1]
+  if (R >= 8) v += lanes_moved<0x141>(v);   // row_half_mirror: lane i of eight with lane 7 - i, which holds the other quad's sum
+  if (R >= 16) v += lanes_moved<0x140>(v);  // row_mirror: lane i of sixteen with lane 15 - i
+#pragma unroll
+  for (int off = 16; off < R; off <<= 1) v += __shfl_xor(v, off, VELOX_WAVE);
+  return v;
+}
 
 struct ScanArgs {
   const float* qk;       // [T, kv_heads, 2, dim]
@@ -441,9 +569,7 @@ __device__ __forceinline__ float scan_token(float (&s)[SCAN_ROWS], const float (
   }
   float u = val;
   if (delta) {
-    float dot = (d[0] + d[1]) + (d[2] + d[3]);
-#pragma unroll
-    for (int off = 1; off < R; off <<= 1) dot += __shfl_xor(dot, off, VELOX_WAVE);
+    const float dot = sum_over_lanes<R>((d[0] + d[1]) + (d[2] + d[3]));
     u = bet * (val - dot);
   }
   float p[4] = {0.f, 0.f, 0.f, 0.f};
@@ -452,10 +578,7 @@ __device__ __forceinline__ float scan_token(float (&s)[SCAN_ROWS], const float (
     s[i] += k[i] * u;
     p[i & 3] += s[i] * q[i];
   }
-  float o = (p[0] + p[1]) + (p[2] + p[3]);
-#pragma unroll
-  for (int off = 1; off < R; off <<= 1) o += __shfl_xor(o, off, VELOX_WAVE);
-  return o;
+  return sum_over_lanes<R>((p[0] + p[1]) + (p[2] + p[3]));
 }
 
 template <int R>
@@ -598,7 +721,7 @@ __global__ void __launch_bounds__(256) linear_scan_staged_kernel(const ScanArgs 
 #pragma unroll
   for (int i = 0; i < SCAN_ROWS; ++i) s[i] = d0 + i < dim ? S[(size_t)(d0 + i) * vdim] : 0.f;
 
-  float q[SCAN_ROWS], k[SCAN_ROWS], dec[SCAN_ROWS], qn[SCAN_ROWS], kn[SCAN_ROWS], decn[SCAN_ROWS];
+  float q[SCAN_ROWS], k[SCAN_ROWS], dec[SCAN_ROWS], qn[SCAN_ROWS], kn[SCAN_ROWS], decn[SCAN_ROWS];  // two sets of operands, used in turn
   float val, bet, valn = 0.f, betn = 1.f;
   auto fetch = [&](int at, float (&fq)[SCAN_ROWS], float (&fk)[SCAN_ROWS], float (&fd)[SCAN_ROWS], float& fv, float& fb) {
     const float one = stage[at + scalars_at + 1];
@@ -635,13 +758,18 @@ __global__ void __launch_bounds__(256) linear_scan_staged_kernel(const ScanArgs 
     const int count = hi - t0 < block_tokens ? hi - t0 : block_tokens;
     const int at = buffer * block_tokens * stride;
     fetch(at, q, k, dec, val, bet);
-    for (int j = 0; j < count; ++j) {
-      if (j + 1 < count) fetch(at + (j + 1) * stride, qn, kn, decn, valn, betn);
+    int j = 0;
+    for (; j + 1 < count; j += 2) {  // (a token's operands are read from LDS while the token before it is worked)
+      fetch(at + (j + 1) * stride, qn, kn, decn, valn, betn);
+      const float o0 = scan_token<R>(s, q, k, dec, val, bet, a.delta);
+      if (live && r == 0) a.out[((size_t)(t0 + j) * heads + h) * vdim + e] = o0;
+      if (j + 2 < count) fetch(at + (j + 2) * stride, q, k, dec, val, bet);
+      const float o1 = scan_token<R>(s, qn, kn, decn, valn, betn, a.delta);
+      if (live && r == 0) a.out[((size_t)(t0 + j + 1) * heads + h) * vdim + e] = o1;
+    }
+    if (j < count) {
       const float o = scan_token<R>(s, q, k, dec, val, bet, a.delta);
       if (live && r == 0) a.out[((size_t)(t0 + j) * heads + h) * vdim + e] = o;
-#pragma unroll
-      for (int i = 0; i < SCAN_ROWS; ++i) { q[i] = qn[i]; k[i] = kn[i]; dec[i] = decn[i]; }
-      val = valn; bet = betn;
     }
     if (more) store_block(buffer ^ 1);  // (the buffer that the block before this one was worked from: everyone is past the barrier behind it)
     __syncthreads();
@@ -657,6 +785,175 @@ extern "C" int velox_linear_scan_lanes(int dim) {
   int lanes = 1;
   while (lanes * SCAN_ROWS < dim) lanes <<= 1;
   return lanes;
+}
+
+// The sum over a wave, the same bits in every lane: rows of 16 as in sum_over_lanes, then row 0's sum into row 1 and row 2's
+// into row 3, the first half's into the second, and the last lane's total to everyone.
+__device__ __forceinline__ float wave_total(float v) {
+  v += lanes_moved<0xB1>(v);
+  v += lanes_moved<0x4E>(v);
+  v += lanes_moved<0x141>(v);
+  v += lanes_moved<0x140>(v);
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x142, 0xA, 0xF, false));  // row_bcast:15, rows 1 and 3 take it
+  v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x143, 0xC, 0xF, false));  // row_bcast:31, rows 2 and 3 take it
+  return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
+}
+
+// linear_scan_wave_kernel: portions of prompts where dim = 64 * RW.  A column of the state is one wave, lane l holds rows
+// l * RW .. l * RW + RW - 1: a token costs a lane 3 RW multiply-adds and two sums over the wave, and a head of 128 x 128 is
+// 128 waves, so that a long prompt of one request still reaches every compute unit.  A workgroup of 512 lanes holds eight
+// columns and stages its head's tokens through LDS as linear_scan_staged_kernel does.  (It reads and writes a column of
+// the state with a stride of vdim floats, once per portion; single tokens keep the kernel whose lanes lie along the rows.)
+#define WAVE_COLS 8
+template <int RW>
+__global__ void __launch_bounds__(512) linear_scan_wave_kernel(const ScanArgs a, const int block_tokens) {
+  extern __shared__ float4_t stage_pieces[];
+  float* stage = reinterpret_cast<float*>(stage_pieces);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int e = blockIdx.x * WAVE_COLS + wave;
+  const int h = blockIdx.y, b = blockIdx.z;
+  const int lo = a.cu_q[b], hi = a.cu_q[b + 1];
+  if (hi <= lo) return;  // (the whole workgroup)
+  const bool live = e < a.vdim;
+  const int col = live ? e : a.vdim - 1;
+  const int dim = 64 * RW, vdim = a.vdim, heads = a.heads;
+  const int d0 = lane * RW;
+  const int g = h / (heads / a.kv_heads);
+  const int per_channel = a.decay_per_channel;
+  const int qk_pieces = dim / 2;
+  const int pieces_per_token = qk_pieces + (per_channel ? dim / 4 : 0);
+  const int values_at = 2 * dim + (per_channel ? dim : 0);
+  const int scalars_at = values_at + WAVE_COLS;
+  const int stride = scalars_at + 4;
+
+  int piece_token[STAGE_PIECES], piece_from[STAGE_PIECES], piece_to[STAGE_PIECES];
+#pragma unroll
+  for (int p = 0; p < STAGE_PIECES; ++p) {
+    const int index = tid + p * 512;
+    const int token = index / pieces_per_token, piece = index - token * pieces_per_token;
+    piece_token[p] = token < block_tokens ? token : -1;
+    piece_from[p] = piece < qk_pieces ? piece * 4 : -1 - (piece - qk_pieces) * 4;
+    piece_to[p] = token * stride + piece * 4;
+  }
+  float4_t carried[STAGE_PIECES];
+  float carried_value = 0.f, carried_beta = 1.f, carried_decay = 1.f;
+  const int value_token = tid / WAVE_COLS, value_col = tid % WAVE_COLS;  // (512 lanes: up to 64 tokens of eight values)
+  auto load_block = [&](int t0) {
+#pragma unroll
+    for (int p = 0; p < STAGE_PIECES; ++p) {
+      const int t = t0 + piece_token[p];
+      if (piece_token[p] >= 0 && t < hi) {
+        const float* from = piece_from[p] >= 0 ? a.qk + ((size_t)t * a.kv_heads + g) * 2 * dim + piece_from[p]
+                                               : a.decay + ((size_t)t * heads + h) * dim + (-1 - piece_from[p]);
+        carried[p] = *reinterpret_cast<const float4_t*>(from);
+      }
+    }
+    if (value_token < block_tokens && t0 + value_token < hi) {
+      const int column = blockIdx.x * WAVE_COLS + value_col;
+      carried_value = column < vdim ? load_as_f32(a.v, a.v_bf16, (size_t)(t0 + value_token) * a.v_ld + a.v_at + (size_t)h * vdim + column) : 0.f;
+    }
+    if (tid < block_tokens && t0 + tid < hi) {
+      carried_beta = a.beta ? a.beta[(size_t)(t0 + tid) * heads + h] : 1.f;
+      carried_decay = per_channel ? 1.f : a.decay[(size_t)(t0 + tid) * heads + h];
+    }
+  };
+  auto store_block = [&](int buffer) {
+    const int at = buffer * block_tokens * stride;
+#pragma unroll
+    for (int p = 0; p < STAGE_PIECES; ++p)
+      if (piece_token[p] >= 0) *reinterpret_cast<float4_t*>(&stage[at + piece_to[p]]) = carried[p];
+    if (value_token < block_tokens) stage[at + value_token * stride + values_at + value_col] = carried_value;
+    if (tid < block_tokens) {
+      stage[at + tid * stride + scalars_at] = carried_beta;
+      stage[at + tid * stride + scalars_at + 1] = carried_decay;
+    }
+  };
+#pragma unroll
+  for (int p = 0; p < STAGE_PIECES; ++p) carried[p] = float4_t{0.f, 0.f, 0.f, 0.f};
+
+  float* S = a.state + (((size_t)a.slots[b] * heads + h) * dim) * vdim + col;
+  float s[RW];
+#pragma unroll
+  for (int i = 0; i < RW; ++i) s[i] = S[(size_t)(d0 + i) * vdim];
+
+  float q[RW], k[RW], dec[RW], qn[RW], kn[RW], decn[RW];  // two sets of operands, used in turn
+  float val, bet, valn = 0.f, betn = 1.f;
+  auto fetch = [&](int at, float (&fq)[RW], float (&fk)[RW], float (&fd)[RW], float& fv, float& fb) {
+    const float one = stage[at + scalars_at + 1];
+#pragma unroll
+    for (int i = 0; i < RW; ++i) {
+      fq[i] = stage[at + d0 + i];
+      fk[i] = stage[at + dim + d0 + i];
+      fd[i] = per_channel ? stage[at + 2 * dim + d0 + i] : one;
+    }
+    fv = stage[at + values_at + wave];
+    fb = stage[at + scalars_at];
+  };
+  auto work = [&](const float (&wq)[RW], const float (&wk)[RW], const float (&wd)[RW], float wv, float wb) -> float {
+    float dot = 0.f;
+#pragma unroll
+    for (int i = 0; i < RW; ++i) {
+      s[i] *= wd[i];
+      dot += s[i] * wk[i];
+    }
+    float u = wv;
+    if (a.delta) u = wb * (wv - wave_total(dot));
+    float part = 0.f;
+#pragma unroll
+    for (int i = 0; i < RW; ++i) {
+      s[i] += wk[i] * u;
+      part += s[i] * wq[i];
+    }
+    return wave_total(part);
+  };
+
+  // Read-outs of a block wait in LDS and leave for memory at the start of the next block, BEFORE that block's loads are
+  // issued: waiting for loads means waiting for every store issued before them too, and a store issued just now is a round
+  // trip to memory, which would then be paid once per block.
+  const int outs_at = 2 * block_tokens * stride;
+  auto flush = [&](int which, int t0, int count) {
+    if (tid < count * WAVE_COLS) {
+      const int token = tid / WAVE_COLS, c = tid % WAVE_COLS;
+      const int column = blockIdx.x * WAVE_COLS + c;
+      if (column < vdim) a.out[((size_t)(t0 + token) * heads + h) * vdim + column] = stage[outs_at + which * block_tokens * WAVE_COLS + tid];
+    }
+  };
+  load_block(lo);
+  store_block(0);
+  __syncthreads();
+  int buffer = 0;
+  for (int t0 = lo; t0 < hi; t0 += block_tokens, buffer ^= 1) {
+    if (t0 > lo) flush(buffer ^ 1, t0 - block_tokens, block_tokens);
+    const bool more = t0 + block_tokens < hi;
+    if (more) load_block(t0 + block_tokens);
+    const int count = hi - t0 < block_tokens ? hi - t0 : block_tokens;
+    const int at = buffer * block_tokens * stride;
+    float* outs = stage + outs_at + buffer * block_tokens * WAVE_COLS + wave;
+    fetch(at, q, k, dec, val, bet);
+    int j = 0;
+    for (; j + 1 < count; j += 2) {  // (a token's operands leave LDS while the token before it is worked)
+      fetch(at + (j + 1) * stride, qn, kn, decn, valn, betn);
+      const float o0 = work(q, k, dec, val, bet);
+      if (j + 2 < count) fetch(at + (j + 2) * stride, q, k, dec, val, bet);
+      const float o1 = work(qn, kn, decn, valn, betn);
+      if (lane == 0) { outs[j * WAVE_COLS] = o0; outs[(j + 1) * WAVE_COLS] = o1; }
+    }
+    if (j < count) {
+      const float o = work(q, k, dec, val, bet);
+      if (lane == 0) outs[j * WAVE_COLS] = o;
+    }
+    if (more) store_block(buffer ^ 1);
+    __syncthreads();
+  }
+  {
+    const int blocks = (hi - lo + block_tokens - 1) / block_tokens;
+    const int last = lo + (blocks - 1) * block_tokens;
+    flush((blocks - 1) & 1, last, hi - last);
+  }
+  if (live) {
+#pragma unroll
+    for (int i = 0; i < RW; ++i) S[(size_t)(d0 + i) * vdim] = s[i];
+  }
 }
 
 // Tokens per staging block: as many as the lanes can carry and two buffers of LDS can hold, 16 at most; 0: no staging.
@@ -680,6 +977,20 @@ extern "C" int velox_linear_scan(const float* qk, const void* v, int v_dtype, in
   ScanArgs a{qk, v, v_dtype == VELOX_BF16, v_ld, v_at, decay, decay_per_channel, beta, state, slots, cu_q, out, heads, kv_heads, dim, vdim, delta};
   const int cols = 256 / lanes;
   const dim3 grid((vdim + cols - 1) / cols, heads, num_seqs);
+  if (max_q_len > 2 && (dim == 64 || dim == 128 || dim == 256 || dim == 512)) {
+    const int stride = 2 * dim + (decay_per_channel ? dim : 0) + WAVE_COLS + 4;
+    int tokens = 16;
+    while (2 * tokens * stride * (int)sizeof(float) > 60 * 1024) tokens >>= 1;  // (dim = 512 with a decay per channel: 4)
+    const size_t lds = (size_t)2 * tokens * (stride + WAVE_COLS) * sizeof(float);  // (two staging buffers, two blocks of read-outs)
+    const dim3 wave_grid((vdim + WAVE_COLS - 1) / WAVE_COLS, heads, num_seqs);
+    switch (dim) {
+      case 64: linear_scan_wave_kernel<1><<<wave_grid, 512, lds, stream>>>(a, tokens); break;
+      case 128: linear_scan_wave_kernel<2><<<wave_grid, 512, lds, stream>>>(a, tokens); break;
+      case 256: linear_scan_wave_kernel<4><<<wave_grid, 512, lds, stream>>>(a, tokens); break;
+      default: linear_scan_wave_kernel<8><<<wave_grid, 512, lds, stream>>>(a, tokens); break;
+    }
+    VELOX_RETURN_LAUNCH_STATUS();
+  }
   const int block_tokens = max_q_len > 2 ? scan_block_tokens(dim, lanes, decay_per_channel) : 0;
   if (block_tokens > 0) {
     const int stride = 2 * dim + (decay_per_channel ? dim : 0) + cols + 4;

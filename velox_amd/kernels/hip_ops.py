@@ -917,7 +917,7 @@ class HipOps:
     def linear_scan_supports(self, dim: int, vdim: int) -> None:
         """Raises if the scan kernel cannot hold a column of a ``dim x vdim`` state in one wave."""
         if self._core.velox_linear_scan_lanes(int(dim)) > 64:
-            raise KernelError(f"linear_scan: key heads of {dim} channels are beyond the kernel (1024 at most)")
+            raise KernelError(f"linear_scan: key heads of {dim} channels are beyond the kernel (512 at most)")
 
     def linear_scan(self, qk, v_source, v_at, decay, beta, state, slots, cu_q, max_q_len, heads, kv_heads, dim, vdim, delta):
         """Per sequence and head, token by token from ``state[slot, head]`` ([dim, vdim] float32), which is written back:
