@@ -805,6 +805,30 @@ __device__ __forceinline__ float wave_total(float v) {
 // columns and stages its head's tokens through LDS as linear_scan_staged_kernel does.  (It reads and writes a column of
 // the state with a stride of vdim floats, once per portion; single tokens keep the kernel whose lanes lie along the rows.)
 #define WAVE_COLS 8
+// 16, 4 or 2 bytes per lane from global memory straight into LDS: lane l's piece lands at `to` + 16 l (4 l for the small
+// ones; two bytes arrive as a zero-extended word).  `to` is the same for the whole wave and is taken from its first
+// active lane.  Assembly, as load_to_lds_16 of common.h and for its reason: the compiler neither moves such a load nor
+// waits for it; the caller waits (wait_for_loads) and places a barrier before anyone reads.
+__device__ __forceinline__ uint32_t lds_address_of_wave(const void* to) {
+  return (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(uintptr_t)(__attribute__((address_space(3))) const char*)to);
+}
+__device__ __forceinline__ void send_to_lds_16(const void* src, const void* to) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(lds_address_of_wave(to)), "v"(src) : "memory", "m0");
+}
+__device__ __forceinline__ void send_to_lds_4(const void* src, const void* to) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" : : "s"(lds_address_of_wave(to)), "v"(src) : "memory", "m0");
+}
+__device__ __forceinline__ void send_to_lds_2(const void* src, const void* to) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_ushort %1, off" : : "s"(lds_address_of_wave(to)), "v"(src) : "memory", "m0");
+}
+
+// A staging buffer of linear_scan_wave_kernel, in floats: q and k of the block's tokens [tokens, 2 dim], the decays per channel
+// [tokens, dim] if there are such, the values of the workgroup's columns [tokens, 8] as they lie in memory (float32, or
+// bfloat16 in the low half of a word), beta [tokens] and the head's decay [tokens].
+__host__ __device__ __forceinline__ int wave_buffer_floats(int tokens, int dim, int per_channel) {
+  return tokens * (2 * dim + (per_channel ? dim : 0) + WAVE_COLS + 2);
+}
+
 template <int RW>
 __global__ void __launch_bounds__(512) linear_scan_wave_kernel(const ScanArgs a, const int block_tokens) {
   extern __shared__ float4_t stage_pieces[];
@@ -820,56 +844,42 @@ __global__ void __launch_bounds__(512) linear_scan_wave_kernel(const ScanArgs a,
   const int d0 = lane * RW;
   const int g = h / (heads / a.kv_heads);
   const int per_channel = a.decay_per_channel;
-  const int qk_pieces = dim / 2;
-  const int pieces_per_token = qk_pieces + (per_channel ? dim / 4 : 0);
-  const int values_at = 2 * dim + (per_channel ? dim : 0);
-  const int scalars_at = values_at + WAVE_COLS;
-  const int stride = scalars_at + 4;
+  const int qk_pieces = dim / 2, decay_pieces = dim / 4;  // 16-byte pieces of a token's q and k, of its decays
+  const int decays_at = block_tokens * 2 * dim;
+  const int values_at = decays_at + (per_channel ? block_tokens * dim : 0);
+  const int betas_at = values_at + block_tokens * WAVE_COLS;
+  const int head_decays_at = betas_at + block_tokens;
+  const int buffer_floats = wave_buffer_floats(block_tokens, dim, per_channel);
 
-  int piece_token[STAGE_PIECES], piece_from[STAGE_PIECES], piece_to[STAGE_PIECES];
-#pragma unroll
-  for (int p = 0; p < STAGE_PIECES; ++p) {
-    const int index = tid + p * 512;
-    const int token = index / pieces_per_token, piece = index - token * pieces_per_token;
-    piece_token[p] = token < block_tokens ? token : -1;
-    piece_from[p] = piece < qk_pieces ? piece * 4 : -1 - (piece - qk_pieces) * 4;
-    piece_to[p] = token * stride + piece * 4;
-  }
-  float4_t carried[STAGE_PIECES];
-  float carried_value = 0.f, carried_beta = 1.f, carried_decay = 1.f;
-  const int value_token = tid / WAVE_COLS, value_col = tid % WAVE_COLS;  // (512 lanes: up to 64 tokens of eight values)
-  auto load_block = [&](int t0) {
-#pragma unroll
-    for (int p = 0; p < STAGE_PIECES; ++p) {
-      const int t = t0 + piece_token[p];
-      if (piece_token[p] >= 0 && t < hi) {
-        const float* from = piece_from[p] >= 0 ? a.qk + ((size_t)t * a.kv_heads + g) * 2 * dim + piece_from[p]
-                                               : a.decay + ((size_t)t * heads + h) * dim + (-1 - piece_from[p]);
-        carried[p] = *reinterpret_cast<const float4_t*>(from);
+  // Sends for the block of tokens from t0: every wave instruction fills 64 consecutive pieces of LDS, each lane from its own
+  // place in memory.  Lanes whose token lies beyond the sequence's end send nothing (nobody reads those rows).
+  auto send_block = [&](int which, int t0) {
+    float* to = stage + which * buffer_floats;
+    for (int first = wave * 64; first < block_tokens * qk_pieces; first += 512) {
+      const int index = first + lane, token = index / qk_pieces, piece = index - token * qk_pieces;
+      if (token < block_tokens && t0 + token < hi)
+        send_to_lds_16(a.qk + ((size_t)(t0 + token) * a.kv_heads + g) * 2 * dim + piece * 4, to + first * 4);
+    }
+    if (per_channel) {
+      for (int first = wave * 64; first < block_tokens * decay_pieces; first += 512) {
+        const int index = first + lane, token = index / decay_pieces, piece = index - token * decay_pieces;
+        if (token < block_tokens && t0 + token < hi)
+          send_to_lds_16(a.decay + ((size_t)(t0 + token) * heads + h) * dim + piece * 4, to + decays_at + first * 4);
       }
     }
-    if (value_token < block_tokens && t0 + value_token < hi) {
-      const int column = blockIdx.x * WAVE_COLS + value_col;
-      carried_value = column < vdim ? load_as_f32(a.v, a.v_bf16, (size_t)(t0 + value_token) * a.v_ld + a.v_at + (size_t)h * vdim + column) : 0.f;
+    for (int first = wave * 64; first < block_tokens * WAVE_COLS; first += 512) {
+      const int index = first + lane, token = index / WAVE_COLS, column = blockIdx.x * WAVE_COLS + index % WAVE_COLS;
+      if (token < block_tokens && t0 + token < hi && column < vdim) {
+        const size_t at = (size_t)(t0 + token) * a.v_ld + a.v_at + (size_t)h * vdim + column;
+        if (a.v_bf16) send_to_lds_2((const bf16_t*)a.v + at, to + values_at + first);
+        else send_to_lds_4((const float*)a.v + at, to + values_at + first);
+      }
     }
-    if (tid < block_tokens && t0 + tid < hi) {
-      carried_beta = a.beta ? a.beta[(size_t)(t0 + tid) * heads + h] : 1.f;
-      carried_decay = per_channel ? 1.f : a.decay[(size_t)(t0 + tid) * heads + h];
-    }
-  };
-  auto store_block = [&](int buffer) {
-    const int at = buffer * block_tokens * stride;
-#pragma unroll
-    for (int p = 0; p < STAGE_PIECES; ++p)
-      if (piece_token[p] >= 0) *reinterpret_cast<float4_t*>(&stage[at + piece_to[p]]) = carried[p];
-    if (value_token < block_tokens) stage[at + value_token * stride + values_at + value_col] = carried_value;
-    if (tid < block_tokens) {
-      stage[at + tid * stride + scalars_at] = carried_beta;
-      stage[at + tid * stride + scalars_at + 1] = carried_decay;
+    if (wave == 7 && lane < block_tokens && t0 + lane < hi) {  // (at most 16 tokens to a block: one wave instruction each)
+      if (a.beta) send_to_lds_4(a.beta + (size_t)(t0 + lane) * heads + h, to + betas_at);
+      if (!per_channel) send_to_lds_4(a.decay + (size_t)(t0 + lane) * heads + h, to + head_decays_at);
     }
   };
-#pragma unroll
-  for (int p = 0; p < STAGE_PIECES; ++p) carried[p] = float4_t{0.f, 0.f, 0.f, 0.f};
 
   float* S = a.state + (((size_t)a.slots[b] * heads + h) * dim) * vdim + col;
   float s[RW];
@@ -878,16 +888,18 @@ __global__ void __launch_bounds__(512) linear_scan_wave_kernel(const ScanArgs a,
 
   float q[RW], k[RW], dec[RW], qn[RW], kn[RW], decn[RW];  // two sets of operands, used in turn
   float val, bet, valn = 0.f, betn = 1.f;
-  auto fetch = [&](int at, float (&fq)[RW], float (&fk)[RW], float (&fd)[RW], float& fv, float& fb) {
-    const float one = stage[at + scalars_at + 1];
+  const int has_beta = a.beta != nullptr, v_bf16 = a.v_bf16;
+  auto fetch = [&](const float* from, int j, float (&fq)[RW], float (&fk)[RW], float (&fd)[RW], float& fv, float& fb) {
+    const float one = per_channel ? 1.f : from[head_decays_at + j];
 #pragma unroll
     for (int i = 0; i < RW; ++i) {
-      fq[i] = stage[at + d0 + i];
-      fk[i] = stage[at + dim + d0 + i];
-      fd[i] = per_channel ? stage[at + 2 * dim + d0 + i] : one;
+      fq[i] = from[j * 2 * dim + d0 + i];
+      fk[i] = from[j * 2 * dim + dim + d0 + i];
+      fd[i] = per_channel ? from[decays_at + j * dim + d0 + i] : one;
     }
-    fv = stage[at + values_at + wave];
-    fb = stage[at + scalars_at];
+    const float raw = from[values_at + j * WAVE_COLS + wave];
+    fv = v_bf16 ? __uint_as_float(__float_as_uint(raw) << 16) : raw;
+    fb = has_beta ? from[betas_at + j] : 1.f;
   };
   auto work = [&](const float (&wq)[RW], const float (&wk)[RW], const float (&wd)[RW], float wv, float wb) -> float {
     float dot = 0.f;
@@ -907,10 +919,8 @@ __global__ void __launch_bounds__(512) linear_scan_wave_kernel(const ScanArgs a,
     return wave_total(part);
   };
 
-  // Read-outs of a block wait in LDS and leave for memory at the start of the next block, BEFORE that block's loads are
-  // issued: waiting for loads means waiting for every store issued before them too, and a store issued just now is a round
-  // trip to memory, which would then be paid once per block.
-  const int outs_at = 2 * block_tokens * stride;
+  // Read-outs of a block wait in LDS and leave for memory at the start of the next block.
+  const int outs_at = 2 * buffer_floats;
   auto flush = [&](int which, int t0, int count) {
     if (tid < count * WAVE_COLS) {
       const int token = tid / WAVE_COLS, c = tid % WAVE_COLS;
@@ -918,23 +928,22 @@ __global__ void __launch_bounds__(512) linear_scan_wave_kernel(const ScanArgs a,
       if (column < vdim) a.out[((size_t)(t0 + token) * heads + h) * vdim + column] = stage[outs_at + which * block_tokens * WAVE_COLS + tid];
     }
   };
-  load_block(lo);
-  store_block(0);
+  send_block(0, lo);
+  wait_for_loads<0>();
   __syncthreads();
   int buffer = 0;
   for (int t0 = lo; t0 < hi; t0 += block_tokens, buffer ^= 1) {
     if (t0 > lo) flush(buffer ^ 1, t0 - block_tokens, block_tokens);
-    const bool more = t0 + block_tokens < hi;
-    if (more) load_block(t0 + block_tokens);
+    if (t0 + block_tokens < hi) send_block(buffer ^ 1, t0 + block_tokens);  // (into the buffer that everyone left at the last barrier)
     const int count = hi - t0 < block_tokens ? hi - t0 : block_tokens;
-    const int at = buffer * block_tokens * stride;
+    const float* from = stage + buffer * buffer_floats;
     float* outs = stage + outs_at + buffer * block_tokens * WAVE_COLS + wave;
-    fetch(at, q, k, dec, val, bet);
+    fetch(from, 0, q, k, dec, val, bet);
     int j = 0;
     for (; j + 1 < count; j += 2) {  // (a token's operands leave LDS while the token before it is worked)
-      fetch(at + (j + 1) * stride, qn, kn, decn, valn, betn);
+      fetch(from, j + 1, qn, kn, decn, valn, betn);
       const float o0 = work(q, k, dec, val, bet);
-      if (j + 2 < count) fetch(at + (j + 2) * stride, q, k, dec, val, bet);
+      if (j + 2 < count) fetch(from, j + 2, q, k, dec, val, bet);
       const float o1 = work(qn, kn, decn, valn, betn);
       if (lane == 0) { outs[j * WAVE_COLS] = o0; outs[(j + 1) * WAVE_COLS] = o1; }
     }
@@ -942,7 +951,7 @@ __global__ void __launch_bounds__(512) linear_scan_wave_kernel(const ScanArgs a,
       const float o = work(q, k, dec, val, bet);
       if (lane == 0) outs[j * WAVE_COLS] = o;
     }
-    if (more) store_block(buffer ^ 1);
+    wait_for_loads<0>();  // this wave's pieces of the next block have landed (and its stores of read-outs, long since)
     __syncthreads();
   }
   {
@@ -978,10 +987,9 @@ extern "C" int velox_linear_scan(const float* qk, const void* v, int v_dtype, in
   const int cols = 256 / lanes;
   const dim3 grid((vdim + cols - 1) / cols, heads, num_seqs);
   if (max_q_len > 2 && (dim == 64 || dim == 128 || dim == 256 || dim == 512)) {
-    const int stride = 2 * dim + (decay_per_channel ? dim : 0) + WAVE_COLS + 4;
     int tokens = 16;
-    while (2 * tokens * stride * (int)sizeof(float) > 60 * 1024) tokens >>= 1;  // (dim = 512 with a decay per channel: 4)
-    const size_t lds = (size_t)2 * tokens * (stride + WAVE_COLS) * sizeof(float);  // (two staging buffers, two blocks of read-outs)
+    while (2 * wave_buffer_floats(tokens, dim, decay_per_channel) * (int)sizeof(float) > 60 * 1024) tokens >>= 1;  // (dim = 512 with a decay per channel: 4)
+    const size_t lds = (size_t)2 * (wave_buffer_floats(tokens, dim, decay_per_channel) + tokens * WAVE_COLS) * sizeof(float);  // (+ two blocks of read-outs)
     const dim3 wave_grid((vdim + WAVE_COLS - 1) / WAVE_COLS, heads, num_seqs);
     switch (dim) {
       case 64: linear_scan_wave_kernel<1><<<wave_grid, 512, lds, stream>>>(a, tokens); break;
