@@ -430,7 +430,7 @@ extern "C" int velox_rotate_pad_write(const void* qkv, int ld, void* q_out, cons
 }
 
 // ---------------------------------------------------------------------------------------------
-// recurrence_prepare: one workgroup per token, waves take heads in turn.
+// recurrence_prepare: one workgroup per token (eight in steps of few tokens), waves take heads in turn.
 //   qk float32 [T, kv_heads, 2, dim]: q (unit vector if `unit`, times q_scale), then k (unit vector if `unit`);
 //   decay float32 [T, columns] = exp(-rate[h] * softplus(sign * (z + bias))), h = column / (columns / heads);
 //   beta float32 [T, heads] = sigmoid(b).
@@ -454,7 +454,8 @@ struct PrepareArgs {
 __global__ void __launch_bounds__(256) recurrence_prepare_kernel(const PrepareArgs a) {
   const size_t t = blockIdx.x;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  for (int h = wave; h < 2 * a.kv_heads; h += 4) {
+  const int part = blockIdx.y, parts = gridDim.y;  // (a step of few tokens spreads each token over several workgroups)
+  for (int h = wave + 4 * part; h < 2 * a.kv_heads; h += 4 * parts) {
     const int g = h >> 1, is_k = h & 1;
     const size_t at = t * a.ld + (is_k ? a.k_at : a.q_at) + (size_t)g * a.dim;
     float inv = 1.f;
@@ -469,12 +470,12 @@ __global__ void __launch_bounds__(256) recurrence_prepare_kernel(const PrepareAr
     for (int c = lane; c < a.dim; c += 64) dst[c] = load_as_f32(a.qkv, a.qkv_bf16, at + c) * inv * factor;
   }
   const int per_head = a.columns / a.heads;
-  for (int c = threadIdx.x; c < a.columns; c += blockDim.x) {
+  for (int c = threadIdx.x + part * blockDim.x; c < a.columns; c += blockDim.x * parts) {
     float z = load_as_f32(a.decay_src, a.decay_bf16, t * a.decay_ld + a.decay_at + c);
     if (a.bias) z += a.bias[c];
     a.decay[t * a.columns + c] = expf(-a.rate[c / per_head] * softplus_f32(a.sign * z));
   }
-  if (a.beta)
+  if (a.beta && part == 0)
     for (int h = threadIdx.x; h < a.heads; h += blockDim.x)
       a.beta[t * a.heads + h] = sigmoid_f32(load_as_f32(a.beta_src, a.beta_bf16, t * a.beta_ld + a.beta_at + h));
 }
@@ -487,7 +488,8 @@ extern "C" int velox_recurrence_prepare(const void* qkv, int qkv_dtype, int ld, 
   if (heads < 1 || columns % heads != 0) return (int)hipErrorInvalidValue;
   PrepareArgs a{qkv, qkv_dtype == VELOX_BF16, ld, q_at, k_at, kv_heads, dim, unit, q_scale, decay_src, decay_dtype == VELOX_BF16, decay_ld, decay_at, heads,
                 columns, rate, bias, sign, beta_src, beta_dtype == VELOX_BF16, beta_ld, beta_at, qk, decay, beta};
-  recurrence_prepare_kernel<<<tokens, 256, 0, stream>>>(a);
+  const int parts = tokens <= 64 ? 8 : 1;
+  recurrence_prepare_kernel<<<dim3(tokens, parts), 256, 0, stream>>>(a);
   VELOX_RETURN_LAUNCH_STATUS();
 }
 
