@@ -129,6 +129,19 @@ def test_embedding_copies_and_gated_activation(ops, ref, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("rows", [1, 8, 33, 200, 2048])
+def test_products_with_a_bias_at_every_number_of_rows(ops, ref, dtype, rows):
+    """The attention's projections carry biases: a few rows take the skinny kernels, many rows the matrix library (bfloat16)
+    or exact multiply-adds (float32); the bias is added to the float32 sums before the one rounding in all of them."""
+    g, dt = torch.Generator().manual_seed(rows), DTYPES[dtype]
+    x, w = rnd(g, rows, 256, dtype=dt), rnd(g, 96, 256, dtype=dt, scale=0.1)
+    bias = rnd(g, 96, dtype=torch.bfloat16).float()  # (as a checkpoint in bfloat16 gives it)
+    want = (x.double() @ w.double().t() + bias.double()).float()
+    near(ops.linear(x, w, bias, dt), want, REL[dtype], "with bias")
+    near(ops.linear(x, w, None, dt), want - bias, REL[dtype], "without")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("taps", [1, 2, 3, 4, 7])
 def test_short_convolution_with_its_last_inputs(ops, ref, dtype, taps):
     g, dt = torch.Generator().manual_seed(taps), DTYPES[dtype]
@@ -222,7 +235,7 @@ def test_recurrence_prepare_scan_and_head_norm(ops, ref, dtype, heads, kv_heads,
 
 
 @pytest.mark.parametrize("heads,kv_heads,dim,vdim,per_channel,delta_rule", [(4, 2, 64, 64, True, True), (2, 2, 128, 128, False, True), (3, 3, 32, 48, True, False), (2, 1, 256, 20, True, True),
-                                                                            (1, 1, 128, 9, True, False), (2, 2, 72, 40, False, True)])
+                                                                            (1, 1, 128, 9, True, False), (2, 2, 72, 40, False, True), (1, 1, 512, 16, True, True)])
 def test_a_long_portion_equals_its_pieces_and_its_first_token_is_kept(ops, ref, heads, kv_heads, dim, vdim, per_channel, delta_rule):
     """600 tokens in one step, in pieces (one of a single token, one of two) and against the plain loop; with decays
     close to 1 the first token's write still decides the last read-out."""
