@@ -129,6 +129,24 @@ def test_embedding_copies_and_gated_activation(ops, ref, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("activation", ["silu", "gelu_tanh"])
+@pytest.mark.parametrize("rows", [1, 5, 16, 17, 40, 300])
+def test_gate_up_product_with_its_activation(ops, ref, dtype, activation, rows):
+    """``act(x Wgate^T) * (x Wup^T)``: one kernel for a decode step's few bfloat16 rows, the product and the activation's kernel
+    otherwise; both against the plain formula on the float32 sums."""
+    g, dt = torch.Generator().manual_seed(rows), DTYPES[dtype]
+    inter, width = 176, 192
+    x, w = rnd(g, rows, width, dtype=dt), rnd(g, 2 * inter, width, dtype=dt, scale=0.15)
+    sums = x.double() @ w.double().t()
+    gate, up = sums[:, :inter], sums[:, inter:]
+    if activation == "silu":
+        want = gate * torch.sigmoid(gate) * up
+    else:
+        want = 0.5 * gate * (1.0 + torch.tanh(0.7978845608028654 * (gate + 0.044715 * gate ** 3))) * up
+    near(ops.linear_gated_act(x, w, dt, activation), want.float(), REL[dtype], f"{activation} {rows} rows")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("rows", [1, 8, 33, 200, 2048])
 def test_products_with_a_bias_at_every_number_of_rows(ops, ref, dtype, rows):
     """The attention's projections carry biases: a few rows take the skinny kernels, many rows the matrix library (bfloat16)

@@ -182,6 +182,7 @@ struct RowScale {
   const float* partial;  // [16][blocks] (row m's sums are contiguous), or null: rows are used as they are
   int blocks;
   float inv_width, eps;
+  int act = 0;  // the gate's activation where a kernel stores act(gate) * up: 0 SiLU, 1 the tanh form of GELU
 };
 
 // How a workgroup adds a row's sums: wave v takes the blocks [v * share, (v + 1) * share), lane (g, row) of it every fourth
@@ -288,7 +289,11 @@ __global__ void __launch_bounds__(WAVES * 64) skinny_gemm_kernel(const bf16_t* _
       for (int wv = 1; wv < WAVES; ++wv) up += partial[wv][tile + RTO * CT][l];
       if constexpr (SCALED) up = up * row_scale;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) sum[j] = sum[j] / (1.f + expf(-sum[j])) * up[j];
+      for (int j = 0; j < 4; ++j) {
+        const float z = sum[j];
+        const float act = rs.act == 1 ? 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z))) : z / (1.f + expf(-z));
+        sum[j] = act * up[j];
+      }
     }
     const int rt = tile / CT, ct = tile % CT;
     const int col_m = 16 * ct + (l & 15);           // batch row
@@ -591,13 +596,15 @@ extern "C" int velox_skinny_residual_norm_bf16(const void* a, const void* w, flo
 // pairs: gate/up tile pairs per wave (1 or 2).
 // a_packed != 0: a is in the lanes' order (see packed_row_offset); out_packed (or null; needs n % 64 == 0): room for
 // n / 64 * 1024 elements, the result once more in that order.  Both only with M <= 16.
-extern "C" int velox_skinny_gemm_glu_bf16(const void* a, const void* w, void* out, int m, int n, int k, int waves, int pairs, int packed,
-                                          const float* scale_partial, int scale_blocks, float inv_width, float eps, int a_packed,
-                                          void* out_packed, hipStream_t stream) {
+// act: 0 SiLU, 1 the tanh form of GELU (velox_skinny_gemm_glu_bf16 is the same with SiLU).
+extern "C" int velox_skinny_gemm_glu_act_bf16(const void* a, const void* w, void* out, int m, int n, int k, int waves, int pairs, int packed,
+                                              const float* scale_partial, int scale_blocks, float inv_width, float eps, int a_packed,
+                                              void* out_packed, int act, hipStream_t stream) {
   if (m <= 0 || n <= 0) return 0;
+  if (act != 0 && act != 1) return -1;
   if (k % 64 != 0 || m > 32 || (scale_partial != nullptr && (m > 16 || scale_blocks > ROW_SCALE_BLOCKS))) return -1;
   if ((a_packed || out_packed != nullptr) && (m > 16 || (out_packed != nullptr && n % 64 != 0))) return -1;
-  const RowScale rs{scale_partial, scale_blocks, inv_width, eps};
+  const RowScale rs{scale_partial, scale_blocks, inv_width, eps, act};
   if (scale_partial != nullptr && waves < 8) waves = 8;  // (rows are scaled by the eight-wave kernels)
   if (m <= 16) {
     if (pairs >= 2) {
@@ -609,6 +616,12 @@ extern "C" int velox_skinny_gemm_glu_bf16(const void* a, const void* w, void* ou
   }
   if (waves >= 8) return launch_skinny_glu<2, 2, 8>(a, w, out, m, n, k, packed != 0, rs, a_packed, out_packed, stream);
   return launch_skinny_glu<2, 2, 4>(a, w, out, m, n, k, packed != 0, rs, a_packed, out_packed, stream);
+}
+
+extern "C" int velox_skinny_gemm_glu_bf16(const void* a, const void* w, void* out, int m, int n, int k, int waves, int pairs, int packed,
+                                          const float* scale_partial, int scale_blocks, float inv_width, float eps, int a_packed,
+                                          void* out_packed, hipStream_t stream) {
+  return velox_skinny_gemm_glu_act_bf16(a, w, out, m, n, k, waves, pairs, packed, scale_partial, scale_blocks, inv_width, eps, a_packed, out_packed, 0, stream);
 }
 
 // ---------------------------------------------------------------------------------------------------------------

@@ -121,6 +121,8 @@ class HipOps:
         c.velox_row_scale_apply.argtypes = [_P, _P, _I, _F, _F, _P, _I, _I, _P]
         c.velox_skinny_gemm_bf16.restype = _I
         c.velox_skinny_gemm_glu_bf16.argtypes = [_P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _I, _F, _F, _I, _P, _P]
+        c.velox_skinny_gemm_glu_act_bf16.argtypes = [_P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _I, _F, _F, _I, _P, _I, _P]
+        c.velox_skinny_gemm_glu_act_bf16.restype = _I
         c.velox_skinny_gemm_glu_bf16.restype = _I
         c.velox_skinny_glu_rows_bf16.argtypes = [_P, _P, _P, _I, _I, _I, _I, _P]
         c.velox_skinny_glu_rows_bf16.restype = _I
@@ -672,8 +674,14 @@ class HipOps:
         self._launched(status, "skinny_gemm")
         return out
 
-    def linear_silu_mul(self, x: torch.Tensor, gate_up_weight: torch.Tensor, out_dtype: torch.dtype, waves: Optional[int] = None, pairs: Optional[int] = None, packed: Optional[torch.Tensor] = None) -> torch.Tensor:
-        """``silu(x Wgate^T) * (x Wup^T)`` for ``W = [Wgate; Wup]``.  Decode-sized bfloat16 batches run as one kernel that
+    def linear_gated_act(self, x: torch.Tensor, gate_up_weight: torch.Tensor, out_dtype: torch.dtype, activation: str) -> torch.Tensor:
+        """``act(x Wgate^T) * (x Wup^T)`` for ``W = [Wgate; Wup]`` and ``activation`` ``"silu"`` or ``"gelu_tanh"``: one kernel for
+        decode-sized bfloat16 batches (see ``linear_silu_mul``), else the product followed by the activation's kernel."""
+        return self.linear_silu_mul(x, gate_up_weight, out_dtype, activation=activation)
+
+    def linear_silu_mul(self, x: torch.Tensor, gate_up_weight: torch.Tensor, out_dtype: torch.dtype, waves: Optional[int] = None, pairs: Optional[int] = None, packed: Optional[torch.Tensor] = None,
+                        activation: str = "silu") -> torch.Tensor:
+        """``silu(x Wgate^T) * (x Wup^T)`` for ``W = [Wgate; Wup]`` (``activation="gelu_tanh"``: the tanh form of GELU in SiLU's place).  Decode-sized bfloat16 batches run as one kernel that
         never writes the [M, 2I] product (up to 16 rows on any weight, 17 .. 64 rows on a registered one); everything else
         is the product followed by the SiLU kernel.  ``waves`` and ``pairs`` override the launch shape the wrapper would
         pick (up to 16 rows: waves per workgroup and gate/up tile pairs per wave; 17 .. 64 rows: ``pairs`` = tile pairs per
@@ -689,7 +697,9 @@ class HipOps:
         two_n = gate_up_weight.shape[0]
         fused = (self.use_skinny_gemm and x.dtype == torch.bfloat16 and gate_up_weight.dtype == torch.bfloat16 and out_dtype == torch.bfloat16
                  and m <= 16 and k % 64 == 0 and two_n % 2 == 0 and x.dim() == 2 and gate_up_weight.shape[1] == k)
-        if (not fused and deferred is None and self.use_skinny_gemm and x.dim() == 2 and 16 < m <= 64 and k % 64 == 0 and two_n % 2 == 0
+        if activation not in ("silu", "gelu_tanh"):
+            raise KernelError(f"linear_silu_mul: activation {activation!r} is not built ('silu' or 'gelu_tanh')")
+        if (not fused and activation == "silu" and deferred is None and self.use_skinny_gemm and x.dim() == 2 and 16 < m <= 64 and k % 64 == 0 and two_n % 2 == 0
                 and x.dtype == torch.bfloat16 and gate_up_weight.dtype == torch.bfloat16 and out_dtype == torch.bfloat16
                 and gate_up_weight.shape[1] == k and packed is not None):
             # 17 .. 64 rows: the kernel that streams the packed weight once with the activation as its epilogue
@@ -707,7 +717,8 @@ class HipOps:
                            "skinny_glu_rows")
             return out
         if not fused:
-            return self.silu_mul(self.linear(deferred if deferred is not None else x, operand, None, out_dtype))
+            product = self.linear(deferred if deferred is not None else x, operand, None, out_dtype)
+            return self.silu_mul(product) if activation == "silu" else self.gated_act_mul(product, activation)
         if deferred is not None and packed is None:  # only the kernels of a registered weight scale rows
             x, deferred = self.materialize(deferred), None
         self._check("x", x, align=16)
@@ -720,9 +731,9 @@ class HipOps:
         out = torch.empty((m, n), dtype=out_dtype, device=self.device)
         x_packed = self._packed_rows_of(x, k)
         out_packed = self._room_for_packed_rows(m, n)
-        status = self._core.velox_skinny_gemm_glu_bf16(_ptr(x if x_packed is None else x_packed), _ptr(packed if packed is not None else gate_up_weight), _ptr(out),
-                                                       m, n, k, int(waves), int(pairs), 1 if packed is not None else 0, *self._scale_args(deferred),
-                                                       int(x_packed is not None), _ptr(out_packed), self._stream())
+        status = self._core.velox_skinny_gemm_glu_act_bf16(_ptr(x if x_packed is None else x_packed), _ptr(packed if packed is not None else gate_up_weight), _ptr(out),
+                                                           m, n, k, int(waves), int(pairs), 1 if packed is not None else 0, *self._scale_args(deferred),
+                                                           int(x_packed is not None), _ptr(out_packed), 1 if activation == "gelu_tanh" else 0, self._stream())
         self._launched(status, "skinny_gemm_glu")
         if out_packed is not None:
             out._velox_packed_rows = (out_packed, out._version)

@@ -59,7 +59,11 @@ class GatedMLP(FeedForward):
             act = ops.linear_silu_mul(x, self.operand("gate_up_weight"), ctx.dtype)
         else:
             # gelu_tanh(z) = z / 2 * (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3))), in float32 with one rounding at the store
-            act = ops.gated_act_mul(ops.linear(x, self.operand("gate_up_weight"), None, ctx.dtype), self.activation)
+            fused = getattr(ops, "linear_gated_act", None)  # (one kernel for decode-sized batches where the operations have it)
+            if fused is not None:
+                act = fused(x, self.operand("gate_up_weight"), ctx.dtype, self.activation)
+            else:
+                act = ops.gated_act_mul(ops.linear(x, self.operand("gate_up_weight"), None, ctx.dtype), self.activation)
         return ops.linear(act, self.operand("down_weight"), None, ctx.dtype, partials_ok=partials_ok, residual_norm=sink)
 
 
