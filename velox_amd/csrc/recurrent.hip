@@ -368,10 +368,11 @@ extern "C" int velox_short_conv(const void* x, int ld, int channels, const float
 }
 
 // ---------------------------------------------------------------------------------------------
-// rotate_pad_write: one workgroup per token.  A row of qkv holds `heads` queries and `kv_heads` keys of `dim` channels and
-// `kv_heads` values of `vdim`.  The first 2 * half channels of every query and key head are rotated (channel i with i + half,
-// cos/sin float32 [positions, half]); queries go to q_out [T, heads * D], keys to k_cache [pages, kv_heads, page, D], values
-// to v_cache [pages, kv_heads, D, page]; channels from dim (vdim) to D are zeros.
+// rotate_pad_write: workgroups take a token's heads in turn (queries, keys, then values; one head each in steps of few tokens).  A row
+// of qkv holds `heads` queries and `kv_heads` keys of `dim` channels and `kv_heads` values of `vdim`.  The first 2 * half
+// channels of every query and key head are rotated (channel i with i + half, cos/sin float32 [positions, half]); queries go to
+// q_out [T, heads * D], keys to k_cache [pages, kv_heads, page, D], values to v_cache [pages, kv_heads, D, page]; channels from
+// dim (vdim) to D are zeros.
 // ---------------------------------------------------------------------------------------------
 template <typename T>
 __global__ void __launch_bounds__(256) rotate_pad_write_kernel(const T* __restrict__ qkv, int ld, T* __restrict__ q_out, const int* __restrict__ positions,
@@ -390,26 +391,28 @@ __global__ void __launch_bounds__(256) rotate_pad_write_kernel(const T* __restri
   }
   const float* cs = half > 0 ? cos_t + (size_t)positions[t] * half : nullptr;
   const float* sn = half > 0 ? sin_t + (size_t)positions[t] * half : nullptr;
-  const int all = (heads + (write_kv ? kv_heads : 0)) * D;
-  for (int i = threadIdx.x; i < all; i += blockDim.x) {
-    const int h = i / D, c = i % D;
+  const int all_heads = heads + (write_kv ? 2 * kv_heads : 0);
+  for (int h = blockIdx.y; h < all_heads; h += gridDim.y) {  // (a step of few tokens has a workgroup per head, a long one a few per token)
+    if (h >= heads + kv_heads) {  // a value head
+      const int g = h - heads - kv_heads;
+      const T* values = row + q_size + k_size + g * vdim;
+      for (int c = threadIdx.x; c < D; c += blockDim.x)
+        v_cache[(((size_t)page * kv_heads + g) * D + c) * page_size + offset] = c < vdim ? values[c] : from_f32<T>(0.f);
+      continue;
+    }
     const bool is_q = h < heads;
     const int g = is_q ? h : h - heads;
     const T* src = row + (is_q ? h * dim : q_size + g * dim);
-    float v = 0.f;
-    if (c < dim) {
-      v = to_f32(src[c]);
-      if (c < half) v = v * cs[c] - to_f32(src[c + half]) * sn[c];
-      else if (c < 2 * half) v = v * cs[c - half] + to_f32(src[c - half]) * sn[c - half];
-    }
     T* dst = is_q ? q_out + ((size_t)t * heads + h) * D : k_cache + (((size_t)page * kv_heads + g) * page_size + offset) * D;
-    dst[c] = from_f32<T>(v);
-  }
-  if (!write_kv) return;
-  const T* values = row + q_size + k_size;
-  for (int i = threadIdx.x; i < kv_heads * D; i += blockDim.x) {
-    const int g = i / D, c = i % D;
-    v_cache[(((size_t)page * kv_heads + g) * D + c) * page_size + offset] = c < vdim ? values[g * vdim + c] : from_f32<T>(0.f);
+    for (int c = threadIdx.x; c < D; c += blockDim.x) {
+      float v = 0.f;
+      if (c < dim) {
+        v = to_f32(src[c]);
+        if (c < half) v = v * cs[c] - to_f32(src[c + half]) * sn[c];
+        else if (c < 2 * half) v = v * cs[c - half] + to_f32(src[c - half]) * sn[c - half];
+      }
+      dst[c] = from_f32<T>(v);
+    }
   }
 }
 
@@ -420,12 +423,16 @@ extern "C" int velox_rotate_pad_write(const void* qkv, int ld, void* q_out, cons
   int shift = 0;
   while ((1 << shift) < page_size) ++shift;
   if ((1 << shift) != page_size || 2 * half > dim || dim > D || vdim > D) return (int)hipErrorInvalidValue;
+  const int all_heads = heads + (write_kv ? 2 * kv_heads : 0);
+  const dim3 grid(tokens, tokens <= 256 ? all_heads : (all_heads < 4 ? all_heads : 4));
+  int lanes = (D + 63) / 64 * 64;
+  if (lanes > 256) lanes = 256;
   if (dtype == VELOX_BF16)
-    rotate_pad_write_kernel<bf16_t><<<tokens, 256, 0, stream>>>((const bf16_t*)qkv, ld, (bf16_t*)q_out, positions, cos_t, sin_t, half, slot_mapping,
-                                                                (bf16_t*)k_cache, (bf16_t*)v_cache, heads, kv_heads, dim, vdim, D, shift, write_kv);
+    rotate_pad_write_kernel<bf16_t><<<grid, lanes, 0, stream>>>((const bf16_t*)qkv, ld, (bf16_t*)q_out, positions, cos_t, sin_t, half, slot_mapping,
+                                                              (bf16_t*)k_cache, (bf16_t*)v_cache, heads, kv_heads, dim, vdim, D, shift, write_kv);
   else
-    rotate_pad_write_kernel<float><<<tokens, 256, 0, stream>>>((const float*)qkv, ld, (float*)q_out, positions, cos_t, sin_t, half, slot_mapping,
-                                                               (float*)k_cache, (float*)v_cache, heads, kv_heads, dim, vdim, D, shift, write_kv);
+    rotate_pad_write_kernel<float><<<grid, lanes, 0, stream>>>((const float*)qkv, ld, (float*)q_out, positions, cos_t, sin_t, half, slot_mapping,
+                                                             (float*)k_cache, (float*)v_cache, heads, kv_heads, dim, vdim, D, shift, write_kv);
   VELOX_RETURN_LAUNCH_STATUS();
 }
 
