@@ -75,6 +75,49 @@ class TorchOps:
         out = out * scale if scale != 1.0 else out
         return out.repeat(1, copies) if copies != 1 else out
 
+    def embed_bigram(self, token_ids, table, bigram, scale, buckets, mul_prev, mul_cur, positions, cu_q, slots, state, max_q_len=None):
+        """Row of the table times ``scale`` plus the row of ``bigram`` that (previous token, token) hash to; position 0 reads
+        row ``buckets``; a portion's first token takes the previous one from ``state`` [slots, 1], which then takes the
+        portion's last token."""
+        ids = token_ids.long()
+        previous = torch.roll(ids, 1)
+        starts, ends = cu_q[:-1].long(), cu_q[1:].long()
+        previous[starts] = state[slots.long(), 0].long()
+        rows = (previous * mul_prev + ids * mul_cur) % buckets
+        rows = torch.where(positions.long() == 0, torch.full_like(rows, buckets), rows)
+        state[slots.long(), 0] = ids[ends - 1].to(state.dtype)
+        return table[ids].float() * scale + bigram[rows].float()
+
+    def add_dynamic_tanh(self, residual, delta, weight, bias, alpha, out_dtype, rows=None):
+        """``residual += delta`` (float32; with ``rows`` nothing is changed and only those rows are worked), then
+        ``tanh(alpha x) * weight + bias``."""
+        delta = self._one_delta(delta)
+        if delta is not None and delta.dim() == 3:
+            delta = delta.float().sum(0)
+        if rows is None:
+            if delta is not None:
+                residual += delta.float()
+            x = residual
+        else:
+            x = residual[rows.long()]
+            if delta is not None:
+                x = x + delta[rows.long()].float()
+        return (torch.tanh(alpha.float() * x) * weight.float() + bias.float()).to(out_dtype)
+
+    def scale_(self, x, factor):
+        return x.mul_(factor)
+
+    def activation(self, x, kind):
+        if kind != "relu2":
+            raise ValueError(kind)
+        return torch.relu(x.float()).square().to(x.dtype)
+
+    def linear_act(self, x, weight, out_dtype, kind):
+        """``act(x W^T)``: the activation on the float32 sums, one rounding."""
+        if kind != "relu2":
+            raise ValueError(kind)
+        return torch.relu(x.float() @ weight.float().T).square().to(out_dtype)
+
     def stream_norm(self, residual, terms, scales, mix, out_weights, in_weights, weight, eps, streams, center, out_dtype, rows=None):
         """``residual`` float32 [T, S * H].  With terms: ``x_t <- sum_s mix[s, t] x_s + out[t] * y`` where ``y = sum_i scales[i]
         terms[i]`` (mix None: identity, out None: ones), in place unless ``rows`` is given.  Returns the norm of
@@ -129,8 +172,9 @@ class TorchOps:
                 tail[slot] = u[u.shape[0] - (taps - 1):].to(tail.dtype)
         return out
 
-    def rotate_pad_write(self, qkv, num_heads, num_kv_heads, dim, vdim, cached_dim, positions, cos, sin, slot_mapping, k_cache, v_cache, block_size, write_kv=True):
-        """Rotates the first ``2 * cos.shape[1]`` channels of every q and k head (halves layout), writes k and v into the
+    def rotate_pad_write(self, qkv, num_heads, num_kv_heads, dim, vdim, cached_dim, positions, cos, sin, slot_mapping, k_cache, v_cache, block_size, write_kv=True,
+                         interleaved=False):
+        """Rotates the first ``2 * cos.shape[1]`` channels of every q and k head (halves layout, or pairs (2i, 2i + 1)), writes k and v into the
         pages at ``cached_dim`` channels a head (zeros in the padding) and returns q as [T, heads * cached_dim]."""
         t = qkv.shape[0]
         q_size, k_size = num_heads * dim, num_kv_heads * dim
@@ -142,6 +186,8 @@ class TorchOps:
             c, s_ = cos[positions.long()][:, None, :], sin[positions.long()][:, None, :]
 
             def rotate(x):
+                if interleaved:
+                    return self._rotate(x, c, s_, True)
                 a, b = x[..., :half], x[..., half:2 * half]
                 return torch.cat([a * c - b * s_, b * c + a * s_, x[..., 2 * half:]], -1)
 
@@ -383,35 +429,55 @@ class TorchOps:
             v_cache[pages, 0, :, offsets] = row
         return queries.view(t, num_heads * cached_dim)
 
-    def head_linear(self, x, x_head_stride, x_offset, maps, out, out_head_stride, out_offset, gate=None, gate_offset=0):
+    def latent_write(self, projected, rot_dim, kv_rank, cached_dim, down_offset, positions, cos, sin, interleaved, norm_weight, eps, slot_mapping,
+                     k_cache, v_cache, block_size, q_latent=None):
+        """The cache write of ``latent_rotate_write`` without any queries; ``q_latent = (offset, rank, weight)``: those
+        columns come back RMS-normed with the weight, [T, rank]."""
+        self.latent_rotate_write(projected, 0, 0, rot_dim, kv_rank, cached_dim, down_offset, positions, cos, sin, interleaved, norm_weight, eps,
+                                 slot_mapping, k_cache, v_cache, block_size)
+        if q_latent is None:
+            return None
+        offset, rank, weight = q_latent
+        part = projected[:, offset:offset + rank].float()
+        return (part / torch.sqrt((part * part).mean(-1, keepdim=True) + eps) * weight.float()).to(projected.dtype)
+
+    def head_linear(self, x, x_head_stride, x_offset, maps, out, out_head_stride, out_offset, gate=None, gate_offset=0, gate_per_head=False):
         groups, n, k = maps.shape
         t = x.shape[0]
         for g in range(groups):
             a = x[:, g * x_head_stride + x_offset:g * x_head_stride + x_offset + k].float()
             y = a @ maps[g].float().T
-            if gate is not None:
+            if gate is not None and gate_per_head:
+                y = y * torch.sigmoid(gate[:, gate_offset + g:gate_offset + g + 1].float())
+            elif gate is not None:
                 y = y * torch.sigmoid(gate[:, gate_offset + g * n:gate_offset + (g + 1) * n].float())
             out[:, g * out_head_stride + out_offset:g * out_head_stride + out_offset + n] = y.to(out.dtype)
         return out
 
     # -- routed experts -------------------------------------------------------------------
-    def route_top(self, logits, top, score="sigmoid", renormalize=False, correction=None):
+    def route_top(self, logits, top, score="sigmoid", renormalize=False, correction=None, groups=None, norm_floor=0.0):
         scores = torch.sigmoid(logits.float()) if score == "sigmoid" else torch.softmax(logits.float(), dim=-1)
-        if correction is not None:  # the correction steers the choice only
-            choice = (scores + correction.float()).topk(top, dim=-1).indices
-            weight = scores.gather(-1, choice)
-        else:
-            weight, choice = scores.topk(top, dim=-1)
+        ranked = scores + correction.float() if correction is not None else scores  # the correction steers the choice only
+        if groups is not None:  # only experts of the best groups can be chosen; a group's score: its two largest choice scores
+            count, keep = groups
+            per = ranked.shape[-1] // count
+            grouped = ranked.view(-1, count, per)
+            best = grouped.topk(min(2, per), dim=-1).values.sum(-1).topk(keep, dim=-1).indices
+            allowed = torch.zeros((ranked.shape[0], count), dtype=torch.bool, device=ranked.device).scatter_(1, best, True)
+            ranked = grouped.masked_fill(~allowed[:, :, None], float("-inf")).reshape(ranked.shape)
+        choice = ranked.topk(top, dim=-1).indices
+        weight = scores.gather(-1, choice)
         if renormalize:
-            weight = weight / weight.sum(-1, keepdim=True)
+            weight = weight / (weight.sum(-1, keepdim=True) + norm_floor)
         return choice.to(torch.int32), weight
 
     def routed_experts(self, x, choice, weight, gate_up_weight, down_weight, num_experts, scale_input, shared, out_dtype, workspace=None,
-                       unit=(1.0, float("inf"), 0.0), identity_experts=0, output_norm=None):
+                       unit=(1.0, float("inf"), 0.0), identity_experts=0, output_norm=None, ungated=None):
         alpha, limit, shift = unit
         t, h = x.shape
-        f = gate_up_weight.shape[0] // (2 * num_experts)
-        gate_up = gate_up_weight.view(num_experts, 2 * f, h).float()
+        branches = 1 if ungated else 2
+        f = gate_up_weight.shape[0] // (branches * num_experts)
+        gate_up = gate_up_weight.view(num_experts, branches * f, h).float()
         down = down_weight.view(num_experts, h, f).float()
         out = torch.zeros((t, h), dtype=torch.float32, device=x.device)
         for k in range(choice.shape[1]):  # a token's results are added in the order of its choices
@@ -425,8 +491,12 @@ class TorchOps:
                 w = weight[rows, k:k + 1]
                 a = (x[rows].float() * w).to(x.dtype).float() if scale_input else x[rows].float()
                 both = a @ gate_up[e].T
-                gate, up = both[:, :f].clamp(max=limit), both[:, f:].clamp(min=-limit, max=limit)
-                act = (gate * torch.sigmoid(alpha * gate) * (up + shift)).to(x.dtype).float()
+                if ungated:
+                    assert ungated == "relu2"
+                    act = torch.relu(both).square().to(x.dtype).float()
+                else:
+                    gate, up = both[:, :f].clamp(max=limit), both[:, f:].clamp(min=-limit, max=limit)
+                    act = (gate * torch.sigmoid(alpha * gate) * (up + shift)).to(x.dtype).float()
                 y = act @ down[e].T
                 out[rows] += y if scale_input else y * w
         if shared is not None:
@@ -439,8 +509,9 @@ class TorchOps:
 
     # -- attention over the paged cache -------------------------------------------------
     def paged_attention(self, qkv, num_heads, num_kv_heads, head_dim, k_cache, v_cache, block_size, block_tables, cu_q, kv_lens, max_q_len, max_kv_len, scale, window, all_decode, workspace, splits=None, decode_prefix=0, portions_max_kv_len=None,
-                        distance_bias=None):
-        """``distance_bias``: float32 [heads, L]; the score of a key ``n`` behind the query gets column ``min(n, L - 1)``."""
+                        distance_bias=None, sinks=None):
+        """``distance_bias``: float32 [heads, L]; the score of a key ``n`` behind the query gets column ``min(n, L - 1)``.
+        ``sinks``: float32 [heads]; ``exp(sinks[h])`` joins the denominator of every row of head ``h``."""
         t = qkv.shape[0]
         group = num_heads // num_kv_heads
         q_all = qkv[:, : num_heads * head_dim].view(t, num_heads, head_dim)
@@ -470,6 +541,8 @@ class TorchOps:
                 m = scores.max(-1, keepdim=True).values
                 p = torch.exp(scores - m)
                 denom = p.sum(-1, keepdim=True)
+                if sinks is not None:
+                    denom = denom + torch.exp(sinks[h].float() - m)
                 p = p.to(qkv.dtype).float()  # the kernel rounds p to the value dtype for the second product
                 out[lo:hi, h] = (p @ values[:, kv]) / denom
         return out.to(qkv.dtype).view(t, num_heads * head_dim)

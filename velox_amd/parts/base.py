@@ -331,6 +331,11 @@ class PositionEncoding(Part):
 
 
 class Embedding(Part):
+    def cache_need(self):
+        """``StateNeed`` if the embedding keeps something per request (then ``forward`` is handed ``cache=``, its
+        ``StateView``), else None."""
+        return None
+
     def forward(self, token_ids: torch.Tensor, ctx) -> torch.Tensor:
         """int32 ``[T]`` -> the residual stream before the first block, float32 ``[T, H]`` (a fresh tensor: blocks
         update it in place)."""

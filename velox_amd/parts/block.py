@@ -31,8 +31,11 @@ class PreNormBlock(Block):
         self.feed_forward = feed_forward
         self.mixer_norm = mixer_norm
         self.ff_norm = ff_norm
+        self.has_feed_forward = type(feed_forward).__name__ != "NoFeedForward"
 
     def children(self) -> Tuple[Part, ...]:
+        if not self.has_feed_forward:
+            return (self.mixer_norm, self.mixer)  # (no second norm: its tensors do not exist)
         return (self.mixer_norm, self.mixer, self.ff_norm, self.feed_forward)
 
     def input_norm(self) -> Optional[Norm]:
@@ -44,6 +47,8 @@ class PreNormBlock(Block):
         normed = self.mixer_norm.forward(residual, pending, ctx)
         if not getattr(self.mixer, "accepts_deferred", False):
             normed = ctx.ops.materialize(normed)  # (a DeferredNorm becomes a tensor; a tensor stays)
+        if not self.has_feed_forward:
+            return self.mixer.forward(normed, ctx, cache, owns_cache)  # (the mixer's output is what the next norm adds)
         if getattr(self.mixer, "accepts_sink", False):
             mixed = self.mixer.forward(normed, ctx, cache, owns_cache, sink=ResidualSink(residual, self.ff_norm))
         else:

@@ -7,7 +7,8 @@ Beside ``parts.attention`` and ``parts.normed_attention`` this mixer has
   ``y_t = sum_j w[:, j] u_(t - taps + 1 + j)``, zeros before the sequence's start (the last column of ``w`` meets the
   current token).  The last ``taps - 1`` projected rows of a sequence are kept in its state slot, in the run dtype, as
   the projection left them, so a portion's first tokens see exactly what they would have seen in a whole prompt;
-* a rotation of the first ``rotary_dim`` channels of each query and key head only (halves layout, the rest passes);
+* a rotation of the first ``rotary_dim`` channels of each query and key head only (the rest passes), in either layout of
+  the position encoding: channel ``i`` with ``i + rotary_dim / 2`` or channel ``2i`` with ``2i + 1``;
 * its own sizes for query/key heads (``dim``) and value heads (``vdim``), a scale from the configuration, a sliding
   window (``window``: a query at ``i`` sees ``j`` with ``0 <= i - j < window``; pages behind it are given back).
 
@@ -41,8 +42,7 @@ class ConvAttentionMixer(Mixer):
             raise ValueError(f"window={window} must be at least 1")
         if conv_taps < 0:
             raise ValueError("conv_taps must not be negative")
-        if getattr(position, "layout", "halves") != "halves":
-            raise ValueError("this mixer's rotation kernel pairs channels (i, i + rotary_dim / 2)")
+        self.interleaved = getattr(position, "layout", "halves") == "interleaved"
         self.hidden_size = int(hidden_size)
         self.num_heads = int(num_heads)
         self.num_kv_heads = int(num_kv_heads)
@@ -137,6 +137,7 @@ class ConvAttentionMixer(Mixer):
         q = ops.rotate_pad_write(
             qkv, self.num_heads, self.num_kv_heads, self.dim, self.vdim, self.cached_dim, ctx.positions, cos, sin,
             meta.slot_mapping, pages.tensors["k"], pages.tensors["v"], pages.block_size, write_kv=owns_cache,
+            **({"interleaved": True} if self.interleaved else {}),
         )
         attn = ops.paged_attention(
             q, self.num_heads, self.num_kv_heads, self.cached_dim,

@@ -23,6 +23,7 @@ from .base import FeedForward, Param, fused_rows, register_part, single
 
 
 SILU_UNIT = (1.0, float("inf"), 0.0)  # (alpha, limit, shift) of ``silu(gate) * up``
+UNGATED_ACTIVATIONS = ("relu2",)  # activations of a unit without a gate branch
 
 
 class GatedMLP(FeedForward):
@@ -70,6 +71,39 @@ class GatedMLP(FeedForward):
 register_part("feed_forward", "gated_mlp", GatedMLP)
 
 
+class PlainMLP(FeedForward):
+    """``W_down act(W_up x)`` without a gate branch and without biases; ``act`` is ``relu2`` (the square of the rectified
+    value).  The activation is float32 with one rounding at the store."""
+
+    def __init__(self, prefix: str, hidden_size: int, intermediate_size: int, activation: str = "relu2",
+                 names: Tuple[str, str] = ("up_proj.weight", "down_proj.weight")) -> None:
+        super().__init__(prefix)
+        if activation not in UNGATED_ACTIVATIONS:
+            raise ValueError(f"activation {activation!r} is not implemented ({', '.join(UNGATED_ACTIVATIONS)})")
+        self.activation = activation
+        self.names = tuple(names)
+        self.hidden_size = int(hidden_size)
+        self.intermediate_size = int(intermediate_size)
+        self.up_weight: Optional[torch.Tensor] = None
+        self.down_weight: Optional[torch.Tensor] = None
+
+    def params(self) -> Dict[str, Param]:
+        h, i = self.hidden_size, self.intermediate_size
+        return {"up_weight": single(self.names[0], (i, h)), "down_weight": single(self.names[1], (h, i))}
+
+    def prepare_kernels(self, ops) -> None:
+        self.prepare_weight(ops, "up_weight")
+        self.prepare_weight(ops, "down_weight")
+
+    def forward(self, x, ctx, sink=None):
+        ops = ctx.ops
+        act = ops.linear_act(x, self.operand("up_weight"), ctx.dtype, self.activation)
+        return ops.linear(act, self.operand("down_weight"), None, ctx.dtype, partials_ok=True)
+
+
+register_part("feed_forward", "plain_mlp", PlainMLP)
+
+
 class NoFeedForward(FeedForward):
     """A layer without a feed-forward: ``forward`` gives None and the block adds nothing."""
 
@@ -98,13 +132,30 @@ class RoutedExperts(FeedForward):
                  expert_names: Tuple[str, str, str] = ("experts.{e}.gate.weight", "experts.{e}.up.weight", "experts.{e}.down.weight"),
                  router_name: str = "router.weight", shared_prefix: str = "shared.",
                  shared_names: Tuple[str, str, str] = ("gate_proj.weight", "up_proj.weight", "down_proj.weight"),
-                 unit: Tuple[float, float, float] = SILU_UNIT, identity_experts: int = 0, correction_name: Optional[str] = None) -> None:
+                 unit: Tuple[float, float, float] = SILU_UNIT, identity_experts: int = 0, correction_name: Optional[str] = None,
+                 ungated: Optional[str] = None, groups: Optional[Tuple[int, int]] = None, renormalize_floor: float = 0.0) -> None:
         """``unit = (alpha, limit, shift)``: a unit's middle is ``g sigmoid(alpha g) (u + shift)`` with ``g = min(W_gate x,
         limit)`` and ``u = clamp(W_up x, -limit, limit)``; ``(1, inf, 0)`` is ``silu(gate) * up``.  ``identity_experts``: the
         router has that many outputs more than there are units; an identity expert's result is its input (times the
         weight, wherever the weight stands).  ``correction_name``: a float32 vector over all router outputs that is added
-        to the scores for the choice only; the weights are the scores without it."""
+        to the scores for the choice only; the weights are the scores without it.  ``ungated``: the units have no gate
+        branch, ``W_down act(W_up x)`` with this activation (``relu2``); ``expert_names`` then names two tensors (up, down)
+        and ``unit`` is not used.  ``groups = (count, keep)``: the experts form ``count`` equal groups of neighbours, a group's
+        score is the sum of its two largest choice scores, and only experts of the ``keep`` best groups can be chosen.
+        ``renormalize_floor``: added to the sum that renormalised weights are divided by."""
         super().__init__(prefix)
+        if ungated is not None and ungated not in UNGATED_ACTIVATIONS:
+            raise ValueError(f"ungated={ungated!r} is not implemented ({', '.join(UNGATED_ACTIVATIONS)})")
+        self.ungated = ungated
+        if ungated is not None and (identity_experts or shared_intermediate_size):
+            raise ValueError("units without a gate branch come without identity experts and without a shared unit")
+        self.groups = (int(groups[0]), int(groups[1])) if groups else None
+        if self.groups is not None:
+            count, keep = self.groups
+            total = int(num_experts) + int(identity_experts)
+            if count < 1 or total % count != 0 or not 1 <= keep <= count or keep * (total // count) < int(top):
+                raise ValueError(f"groups={groups}: {total} experts must form equal groups, and the kept groups must hold at least top={top} experts")
+        self.renormalize_floor = float(renormalize_floor)
         self.unit = (float(unit[0]), float(unit[1]), float(unit[2]))
         if not self.unit[1] > 0:
             raise ValueError(f"unit: the limit must be positive (inf for none), got {self.unit[1]}")
@@ -135,11 +186,13 @@ class RoutedExperts(FeedForward):
 
     def params(self) -> Dict[str, Param]:
         h, f, e = self.hidden_size, self.intermediate_size, self.num_experts
-        gate, up, down = self.expert_names
-        gate_up_names = tuple(name.format(e=i) for i in range(e) for name in (gate, up))
+        first, down = self.expert_names[:-1], self.expert_names[-1]  # (gate, up) or, without a gate branch, (up,)
+        if len(first) != (1 if self.ungated else 2):
+            raise ValueError(f"expert_names must name {'up and down' if self.ungated else 'gate, up and down'}")
+        gate_up_names = tuple(name.format(e=i) for i in range(e) for name in first)
         out = {
             "router_weight": single(self.router_name, (e + self.identity_experts, h)),
-            "gate_up_weight": fused_rows(gate_up_names, ((f, h),) * (2 * e)),
+            "gate_up_weight": fused_rows(gate_up_names, ((f, h),) * (len(first) * e)),
             "down_weight": fused_rows(tuple(down.format(e=i) for i in range(e)), ((h, f),) * e),
         }
         if self.correction_name is not None:
@@ -161,10 +214,17 @@ class RoutedExperts(FeedForward):
         ops = ctx.ops
         x = ops.materialize(x)
         logits = ops.linear(x, self.router_weight, None, torch.float32)
+        options = {}
         if self.correction is not None:
-            choice, weight = ops.route_top(logits, self.top, self.score, self.renormalize, correction=self.correction)
-        else:
-            choice, weight = ops.route_top(logits, self.top, self.score, self.renormalize)
+            options["correction"] = self.correction
+        if self.groups is not None:
+            options["groups"] = self.groups
+        if self.renormalize_floor:
+            options["norm_floor"] = self.renormalize_floor
+        choice, weight = ops.route_top(logits, self.top, self.score, self.renormalize, **options)
+        if self.ungated is not None:
+            return ops.routed_experts(x, choice, weight, self.gate_up_weight, self.down_weight, self.num_experts, self.scale_input, None,
+                                      ctx.dtype, ctx.workspace, ungated=self.ungated, **({"output_norm": output_norm} if output_norm is not None else {}))
         shared = self.shared.forward(x, ctx, partials_ok=False) if self.shared is not None else None
         if output_norm is not None:
             return ops.routed_experts(x, choice, weight, self.gate_up_weight, self.down_weight, self.num_experts, self.scale_input, shared,

@@ -19,10 +19,14 @@ plain kernel of any size takes their place), and is held
 twice, as keys ``[page, 1, offset, D]`` and transposed as values ``[page, 1, D, offset]``, the layout those
 kernels read (``parts.attention.kv_pages``).
 
-Options of the part: a sigmoid gate on the concatenated heads (``gate``), and ``own_latent`` = False for a layer
+Options of the part: a sigmoid gate on the concatenated heads (``gate``: one number per channel, or ``"head"``: one per
+head), and ``own_latent`` = False for a layer
 that makes no latent of its own and reads another schedule entry's cache (``ScheduleEntry.cache_from``) with its
 own ``U``, ``V``, queries and output product.  The rotation (which channels pair up, the frequencies, a factor on
-cos and sin) is the position encoding's; it is applied to the first ``2 * table width`` channels of the rotated part.
+cos and sin) is the position encoding's; it is applied to the first ``2 * table width`` channels of the rotated part;
+``rot_dim`` = 0 is attention without positions.  ``q_rank``: the queries pass a latent of their own,
+``q = W_uq rmsnorm(W_dq x)``, the norm in float32 inside the kernel that writes the cache.  ``sink``: a learned number per
+head whose exponential joins the softmax's denominator (it has no key and no value and is not scaled).
 """
 from __future__ import annotations
 
@@ -34,15 +38,16 @@ from .attention import SHORT_CONTEXT_KEYS, kv_pages
 from .base import Mixer, Param, PositionEncoding, fused_rows, register_part, single
 
 _NAMES = {"q": "q.weight", "down": "down.weight", "down_norm": "down_norm.weight", "up_k": "up_k.weight", "up_v": "up_v.weight",
-          "gate": "gate.weight", "out": "out.weight"}
+          "gate": "gate.weight", "out": "out.weight", "q_down": "q_down.weight", "q_norm": "q_norm.weight", "q_up": "q_up.weight", "sink": "sink"}
 
 
 class LatentAttentionMixer(Mixer):
     def __init__(self, prefix: str, hidden_size: int, num_heads: int, dim: int, rot_dim: int, vdim: int, kv_rank: int, scale: float,
-                 norm_eps: float, position: Optional[PositionEncoding] = None, gate: bool = True, own_latent: bool = True,
-                 names: Tuple[Tuple[str, str], ...] = ()) -> None:
+                 norm_eps: float, position: Optional[PositionEncoding] = None, gate=True, own_latent: bool = True,
+                 names: Tuple[Tuple[str, str], ...] = (), q_rank: Optional[int] = None, sink: bool = False) -> None:
         """``names``: pairs (role, tensor name below the prefix) that replace the defaults for the roles ``q``, ``down``,
-        ``down_norm``, ``up_k``, ``up_v``, ``gate``, ``out``."""
+        ``down_norm``, ``up_k``, ``up_v``, ``gate``, ``out``, ``q_down``, ``q_norm``, ``q_up``, ``sink``.  ``gate``: False,
+        True (a number per channel of the concatenated heads) or ``"head"`` (a number per head)."""
         super().__init__(prefix)
         for label, value in (("hidden_size", hidden_size), ("num_heads", num_heads), ("dim", dim), ("vdim", vdim), ("kv_rank", kv_rank)):
             if int(value) < 1:
@@ -53,16 +58,25 @@ class LatentAttentionMixer(Mixer):
         self.dim, self.rot_dim, self.vdim, self.kv_rank = int(dim), int(rot_dim), int(vdim), int(kv_rank)
         self.scale, self.norm_eps = float(scale), float(norm_eps)
         self.position = position
+        if gate not in (True, False, "head", "channel"):
+            raise ValueError(f"gate={gate!r} must be False, True, 'channel' or 'head'")
         self.gate, self.own_latent = bool(gate), bool(own_latent)
+        self.gate_per_head = gate == "head"
+        self.q_rank = int(q_rank) if q_rank else 0
+        self.sink = bool(sink)
         self.names = dict(_NAMES)
         self.names.update(dict(names))
         self.cached_dim = (self.kv_rank + self.rot_dim + 15) // 16 * 16
         if self.cached_dim > 1024:
             raise ValueError(f"kv_rank + rot_dim = {self.kv_rank + self.rot_dim}: the attention kernels take at most 1,024 cached channels per token")
         self.q_size = self.num_heads * (self.dim + self.rot_dim)
-        self.gate_size = self.num_heads * self.vdim if self.gate else 0
+        self.gate_size = (self.num_heads if self.gate_per_head else self.num_heads * self.vdim) if self.gate else 0
+        self.first_size = self.q_rank or self.q_size  # what stands first in the rows of the input product: the queries or their latent
         self.down_size = self.kv_rank + self.rot_dim if self.own_latent else 0
-        self.in_weight: Optional[torch.Tensor] = None  # rows [W_q ; W_gate ; W_down]
+        self.in_weight: Optional[torch.Tensor] = None  # rows [W_q (or W_dq) ; W_gate ; W_down]
+        self.q_norm_weight: Optional[torch.Tensor] = None
+        self.q_up_weight: Optional[torch.Tensor] = None  # [heads * (dim + rot_dim), q_rank]
+        self.sink_logits: Optional[torch.Tensor] = None  # float32 [heads]
         self.down_norm_weight: Optional[torch.Tensor] = None
         self.up_k_weight: Optional[torch.Tensor] = None  # [heads * dim, kv_rank]
         self.up_v_weight: Optional[torch.Tensor] = None  # [heads * vdim, kv_rank]
@@ -72,7 +86,7 @@ class LatentAttentionMixer(Mixer):
 
     def params(self) -> Dict[str, Param]:
         h, n = self.hidden_size, self.names
-        sources, shapes = [n["q"]], [(self.q_size, h)]
+        sources, shapes = ([n["q_down"]], [(self.q_rank, h)]) if self.q_rank else ([n["q"]], [(self.q_size, h)])
         if self.gate:
             sources.append(n["gate"])
             shapes.append((self.gate_size, h))
@@ -87,6 +101,11 @@ class LatentAttentionMixer(Mixer):
         }
         if self.own_latent:
             out["down_norm_weight"] = single(n["down_norm"], (self.kv_rank,), role="vector", init="one_plus_normal")
+        if self.q_rank:
+            out["q_norm_weight"] = single(n["q_norm"], (self.q_rank,), role="vector", init="one_plus_normal")
+            out["q_up_weight"] = single(n["q_up"], (self.q_size, self.q_rank))
+        if self.sink:
+            out["sink_logits"] = single(n["sink"], (self.num_heads,), role="vector")
         return out
 
     def cache_need(self):
@@ -111,6 +130,8 @@ class LatentAttentionMixer(Mixer):
             raise ValueError(f"the rotation spans {2 * cos.shape[1]} channels but the rotated part has {self.rot_dim}")
         self.prepare_weight(ops, "in_weight")
         self.prepare_weight(ops, "out_weight")
+        if self.q_rank:
+            self.prepare_weight(ops, "q_up_weight")
 
     def capture_key_bounds(self, ops, batch: int, max_model_len: int):
         choose = getattr(ops, "choose_splits", None)
@@ -132,15 +153,28 @@ class LatentAttentionMixer(Mixer):
             raise ValueError("a latent-attention layer writes the cache exactly when it has a down-projection of its own")
         cos, sin, interleaved = self._rotary()
         meta = cache.batch
-        projected = ops.linear(x, self.operand("in_weight"), None, ctx.dtype)  # [T, q | gate | down]
-        # rotation of the queries' rotated parts; norm of the latent, rotation of the shared key part and their write
-        # into the cache; the rotated query parts land behind the room for U_h^T a_h in the queries the kernels read
-        queries = ops.latent_rotate_write(
-            projected, self.num_heads, self.dim, self.rot_dim, self.kv_rank, self.cached_dim, self.q_size + self.gate_size if self.own_latent else -1,
-            ctx.positions, cos, sin, interleaved, self.down_norm_weight, self.norm_eps,
-            meta.slot_mapping, cache.tensors["k"], cache.tensors["v"], cache.block_size)
+        projected = ops.linear(x, self.operand("in_weight"), None, ctx.dtype)  # [T, q (or its latent) | gate | down]
+        down_offset = self.first_size + self.gate_size if self.own_latent else -1
+        if self.q_rank:
+            # norm of the latent, rotation of the shared key part and their write into the cache; the queries' own latent
+            # is normed by the same kernel and goes through W_uq; then the rotation of the queries' rotated parts
+            q_latent = ops.latent_write(
+                projected, self.rot_dim, self.kv_rank, self.cached_dim, down_offset, ctx.positions, cos, sin, interleaved, self.down_norm_weight, self.norm_eps,
+                meta.slot_mapping, cache.tensors["k"], cache.tensors["v"], cache.block_size, q_latent=(0, self.q_rank, self.q_norm_weight))
+            q_source = ops.linear(q_latent, self.operand("q_up_weight"), None, ctx.dtype)
+            queries = ops.latent_rotate_write(
+                q_source, self.num_heads, self.dim, self.rot_dim, self.kv_rank, self.cached_dim, -1, ctx.positions, cos, sin, interleaved,
+                None, self.norm_eps, None, None, None, cache.block_size)
+        else:
+            # rotation of the queries' rotated parts; norm of the latent, rotation of the shared key part and their write
+            # into the cache; the rotated query parts land behind the room for U_h^T a_h in the queries the kernels read
+            q_source = projected
+            queries = ops.latent_rotate_write(
+                projected, self.num_heads, self.dim, self.rot_dim, self.kv_rank, self.cached_dim, down_offset,
+                ctx.positions, cos, sin, interleaved, self.down_norm_weight, self.norm_eps,
+                meta.slot_mapping, cache.tensors["k"], cache.tensors["v"], cache.block_size)
         # queries[t, h, :kv_rank] = U_h^T a_h(t)
-        ops.head_linear(projected, self.dim + self.rot_dim, 0, self.query_maps, queries, self.cached_dim, 0)
+        ops.head_linear(q_source, self.dim + self.rot_dim, 0, self.query_maps, queries, self.cached_dim, 0)
         attended = ops.paged_attention(
             queries, self.num_heads, 1, self.cached_dim,
             cache.tensors["k"], cache.tensors["v"], cache.block_size,
@@ -148,11 +182,12 @@ class LatentAttentionMixer(Mixer):
             ctx.max_q_len, meta.max_kv_len, self.scale, None,
             ctx.all_decode, ctx.workspace,
             decode_prefix=getattr(ctx, "decode_prefix", 0), portions_max_kv_len=getattr(meta, "max_kv_len_of_portions", 0) or None,
+            **({"sinks": self.sink_logits} if self.sink else {}),
         )
         # heads[t, h] = V_h attended[t, h, :kv_rank], times sigmoid(gate) when the layer has a gate
         heads = torch.empty((x.shape[0], self.num_heads * self.vdim), dtype=ctx.dtype, device=x.device)
         ops.head_linear(attended, self.cached_dim, 0, self.value_maps, heads, self.vdim, 0,
-                        gate=projected if self.gate else None, gate_offset=self.q_size)
+                        gate=projected if self.gate else None, gate_offset=self.first_size, **({"gate_per_head": True} if self.gate_per_head else {}))
         return ops.linear(heads, self.operand("out_weight"), None, ctx.dtype, partials_ok=True)
 
 

@@ -20,7 +20,7 @@ from typing import Dict, List, Optional, Tuple
 import torch
 
 from . import block as _block  # noqa: F401  (registers the built-in arrangement)
-from .base import Embedding, OutputHead, Param, Part, PartSpec, make_part, register_part, single
+from .base import Embedding, OutputHead, Param, Part, PartSpec, StateNeed, make_part, register_part, single
 
 
 @dataclass(frozen=True)
@@ -108,12 +108,47 @@ class TableEmbedding(Embedding):
         return ctx.ops.embed(token_ids, self.table, scale=self.scale)
 
 
-class LinearHead(OutputHead):
-    """``logits = hidden @ W^T`` without bias; ``W`` is the embedding table when tied
-    (reference ``src/transformer.py:60-62``).  Logits are returned in float32."""
+class BigramEmbedding(TableEmbedding):
+    """``h[t] = E[ids[t]] * scale + B[(ids[t-1] * mul_prev + ids[t] * mul_cur) mod buckets]``: beside the token's own row, a
+    row of a second table chosen by a hash of the token and the one before it; a sequence's first token reads the
+    table's last row (row ``buckets``).  The token before a portion's first one is part of the request's state: one
+    int32 per state slot, which the kernel that looks the rows up reads for a portion's first token and sets to the
+    portion's last token (a request at position 0 does not read it).  The sum is float32."""
 
-    def __init__(self, name: str, vocab_size: int, hidden_size: int, tied_to: Optional[str] = None) -> None:
+    def __init__(self, name: str, vocab_size: int, hidden_size: int, buckets: int, mul_prev: int, mul_cur: int, scale: float = 1.0,
+                 bigram_name: str = "bigram") -> None:
+        super().__init__(name, vocab_size, hidden_size, scale)
+        if int(buckets) < 1:
+            raise ValueError(f"buckets={buckets} must be positive")
+        self.buckets, self.mul_prev, self.mul_cur = int(buckets), int(mul_prev), int(mul_cur)
+        self.bigram_name = bigram_name
+        self.bigram: Optional[torch.Tensor] = None
+
+    def params(self) -> Dict[str, Param]:
+        out = super().params()
+        out["bigram"] = single(self.bigram_name, (self.buckets + 1, self.hidden_size), product=False)
+        return out
+
+    def cache_need(self):
+        return StateNeed((("previous_token", (1,), torch.int32),))
+
+    def forward(self, token_ids: torch.Tensor, ctx, copies: int = 1, cache=None) -> torch.Tensor:
+        if copies != 1:
+            raise ValueError("the bigram embedding writes one residual stream")
+        if cache is None:
+            raise ValueError("the bigram embedding needs its state (the token before each portion)")
+        return ctx.ops.embed_bigram(token_ids, self.table, self.bigram, self.scale, self.buckets, self.mul_prev, self.mul_cur,
+                                    ctx.positions, ctx.cu_q, ctx.slots, cache.tensors["previous_token"], ctx.max_q_len)
+
+
+class LinearHead(OutputHead):
+    """``logits = (hidden @ W^T) * scale`` without bias; ``W`` is the embedding table when tied
+    (reference ``src/transformer.py:60-62``; it has no scale, which is ``scale`` = 1).  Logits are returned in float32
+    and the scale is applied to them there."""
+
+    def __init__(self, name: str, vocab_size: int, hidden_size: int, tied_to: Optional[str] = None, scale: float = 1.0) -> None:
         super().__init__("")
+        self.scale = float(scale)
         self.name = name
         self.vocab_size = vocab_size
         self.hidden_size = hidden_size
@@ -130,10 +165,12 @@ class LinearHead(OutputHead):
         self.prepare_weight(ops, "weight")
 
     def forward(self, hidden_rows: torch.Tensor, ctx) -> torch.Tensor:
-        return ctx.ops.linear(hidden_rows, self.operand("weight"), None, torch.float32)
+        logits = ctx.ops.linear(hidden_rows, self.operand("weight"), None, torch.float32)
+        return logits if self.scale == 1.0 else ctx.ops.scale_(logits, self.scale)
 
 
 register_part("embedding", "table", TableEmbedding)
+register_part("embedding", "bigram_table", BigramEmbedding)
 register_part("head", "linear", LinearHead)
 
 
@@ -183,17 +220,25 @@ class DecoderModel(Part):
         return all(part.graph_safe for part in self.all_parts())
 
     def cache_needs(self) -> List[object]:
-        """One entry per schedule entry: the mixer's need, or None when it reads another entry's cache."""
+        """One entry per schedule entry: the mixer's need, or None when it reads another entry's cache.  An embedding
+        that keeps something per request (``Embedding.cache_need``) adds one entry behind the schedule's."""
         needs = []
         for entry in self.schedule:
             need = self.blocks[entry.layer].cache_need()
             needs.append(need if entry.cache_from is None else None)
+        if self.embedding.cache_need() is not None:
+            needs.append(self.embedding.cache_need())
         return needs
 
     # -- arithmetic ---------------------------------------------------------------------
     def embed(self, token_ids: torch.Tensor, ctx) -> torch.Tensor:
         """The residual stream before the first block: float32 ``[T, H]``."""
         streams = self.spec.residual_streams
+        if self.embedding.cache_need() is not None:
+            residual = self.embedding.forward(token_ids, ctx, cache=ctx.cache_view(len(self.schedule)))
+            if self.spec.embedding_position is not None:
+                residual = self.positions[self.spec.embedding_position].on_embeddings(residual, ctx)
+            return residual.repeat(1, streams) if streams > 1 else residual
         if streams > 1 and self.spec.embedding_position is None:
             return self.embedding.forward(token_ids, ctx, copies=streams)  # (the looked-up row written once per stream)
         residual = self.embedding.forward(token_ids, ctx)

@@ -1,4 +1,5 @@
-"""Norms that own the residual update: RMSNorm, and a norm over several residual streams (``StreamNorm``).
+"""Norms that own the residual update: RMSNorm, a norm over several residual streams (``StreamNorm``) and a norm without
+statistics (``DynamicTanhNorm``).
 
 Formula (reference ``src/rmsnorm.py:20-28``): in float32, ``y = x * rsqrt(mean(x^2) + eps) * w``,
 one rounding at the store.  The reference adds the residual in the model dtype
@@ -98,3 +99,37 @@ class StreamNorm(Norm):
 
 
 register_part("norm", "stream_norm", StreamNorm)
+
+
+class DynamicTanhNorm(Norm):
+    """A norm that takes no mean and no variance: ``y = tanh(alpha * x) * w + b`` per channel, with one learned number
+    ``alpha`` for the whole layer, a weight and a bias.  The residual update is the same as for every norm here
+    (``residual += delta`` in float32 inside the norm's kernel); ``alpha`` stays on the device, so the norm reads nothing
+    on the host.  It cannot be split into a product's epilogue and the next product's row scale (there is no row scale).
+
+    ``weight_name``, ``bias_name`` and ``alpha_name`` are the tensors' names below the prefix."""
+
+    def __init__(self, prefix: str, hidden_size: int, weight_name: str = "weight", bias_name: str = "bias", alpha_name: str = "alpha") -> None:
+        super().__init__(prefix)
+        self.hidden_size = int(hidden_size)
+        self.weight_name, self.bias_name, self.alpha_name = weight_name, bias_name, alpha_name
+        self.weight: Optional[torch.Tensor] = None
+        self.bias: Optional[torch.Tensor] = None
+        self.alpha: Optional[torch.Tensor] = None
+
+    def params(self) -> Dict[str, Param]:
+        return {
+            "weight": single(self.weight_name, (self.hidden_size,), role="vector", init="one_plus_normal"),
+            "bias": single(self.bias_name, (self.hidden_size,), role="vector"),
+            "alpha": single(self.alpha_name, (), role="vector", init="one_plus_normal"),
+        }
+
+    def forward(self, residual, delta, ctx, rows=None):
+        if isinstance(delta, DeferredNorm):
+            raise ValueError("this norm cannot be split into a product's epilogue")
+        if isinstance(delta, ResidualCopy):
+            delta = None
+        return ctx.ops.add_dynamic_tanh(residual, delta, self.weight, self.bias, self.alpha, ctx.dtype, rows=rows)
+
+
+register_part("norm", "dynamic_tanh", DynamicTanhNorm)
