@@ -152,7 +152,8 @@ __global__ void __launch_bounds__(64 * WAVES * KSPLIT) __attribute__((amdgpu_wav
     const T* __restrict__ qkv, int qkv_stride, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int* __restrict__ block_tables, int table_width, const int* __restrict__ cu_q, const int* __restrict__ kv_lens,
     T* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_lse,
-    int nh, int nkv, int page_shift, float scale, int window, int splits, int total_tokens, const float* __restrict__ bias_table, int bias_len) {
+    int nh, int nkv, int page_shift, float scale, int window, int splits, int total_tokens, const float* __restrict__ bias_table, int bias_len,
+    const float* __restrict__ sinks) {
   typedef Block<T> B;
   typedef typename B::Operand Operand;
   constexpr int KB = B::KB;
@@ -561,6 +562,8 @@ __global__ void __launch_bounds__(64 * WAVES * KSPLIT) __attribute__((amdgpu_wav
     l += __shfl_xor(l, 16, VELOX_WAVE);
     l += __shfl_xor(l, 32, VELOX_WAVE);
     if (!row_ok[ct]) continue;
+    // a sink joins the denominator once, where nothing is merged later (with split keys: in the merge kernel)
+    if (sinks != nullptr && splits == 1 && l > 0.f) l += Softmax<T>::exp_of(sinks[head[ct]] * Softmax<T>::SCALE - m_i[ct]);
     const float inv = l > 0.f ? 1.f / l : 1.f;
     const size_t token = (size_t)(q_start + tok[ct]);
     if (splits == 1) {
@@ -610,7 +613,8 @@ __global__ void __launch_bounds__(64 * WAVES * KSPLIT) __attribute__((amdgpu_wav
     const bf16_t* __restrict__ qkv, int qkv_stride, const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
     const int* __restrict__ block_tables, int table_width, const int* __restrict__ cu_q, const int* __restrict__ kv_lens,
     bf16_t* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_lse,
-    int nh, int nkv, int page_shift, float scale, int window, int splits, int total_tokens, const float* __restrict__ bias_table, int bias_len) {
+    int nh, int nkv, int page_shift, float scale, int window, int splits, int total_tokens, const float* __restrict__ bias_table, int bias_len,
+    const float* __restrict__ sinks) {
   typedef bf16_t T;
   typedef Block<T> B;
   typedef typename B::Operand Operand;
@@ -1004,6 +1008,8 @@ __global__ void __launch_bounds__(64 * WAVES * KSPLIT) __attribute__((amdgpu_wav
     l += __shfl_xor(l, 16, VELOX_WAVE);
     l += __shfl_xor(l, 32, VELOX_WAVE);
     if (!row_ok[ct]) continue;
+    // a sink joins the denominator once, where nothing is merged later (with split keys: in the merge kernel)
+    if (sinks != nullptr && splits == 1 && l > 0.f) l += Softmax<T>::exp_of(sinks[head[ct]] * Softmax<T>::SCALE - m_i[ct]);
     const float inv = l > 0.f ? 1.f / l : 1.f;
     const size_t token = (size_t)(q_start + tok[ct]);
     if (splits == 1) {
@@ -1068,7 +1074,8 @@ __global__ void __launch_bounds__(64 * WAVES) decode_attention_kernel(
     const T* __restrict__ qkv, int qkv_stride, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int* __restrict__ block_tables, int table_width, const int* __restrict__ kv_lens,
     T* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_lse,
-    int nh, int nkv, int page_shift, float scale, int window, int splits, int total_tokens, const float* __restrict__ bias_table, int bias_len) {
+    int nh, int nkv, int page_shift, float scale, int window, int splits, int total_tokens, const float* __restrict__ bias_table, int bias_len,
+    const float* __restrict__ sinks) {
   constexpr int NC = D / 16;
   constexpr int NCW = (NC + WAVES - 1) / WAVES;
   typedef KeyOps<T, sizeof(T) == 2 && D % 32 == 0> KO;
@@ -1260,6 +1267,7 @@ __global__ void __launch_bounds__(64 * WAVES) decode_attention_kernel(
     l_tot += weight[w] * l_all[w * 16 + i];
   }
   if (!row_ok) return;
+  if (sinks != nullptr && splits == 1 && l_tot > 0.f) l_tot += softmax_exp<T>(sinks[head] - m_ref);  // (see the general kernel)
   const float inv = l_tot > 0.f ? 1.f / l_tot : 1.f;
   const size_t slot = ((size_t)split * total_tokens + b) * nh + head;
 #pragma unroll
@@ -1281,10 +1289,11 @@ __global__ void __launch_bounds__(64 * WAVES) decode_attention_kernel(
   if (splits > 1 && wave == 0 && g == 0) part_lse[slot] = l_tot > 0.f ? m_tot + logf(l_tot) : -INFINITY;
 }
 
-// out[token, head, :] = sum_s w_s * o_s / sum_s w_s,  w_s = exp(lse_s - max_s lse_s)
+// out[token, head, :] = sum_s w_s * o_s / sum_s w_s,  w_s = exp(lse_s - max_s lse_s); a sink adds exp(sink - max_s lse_s)
+// to the denominator
 template <typename T>
 __global__ void merge_splits_kernel(const float* __restrict__ part_o, const float* __restrict__ part_lse, T* __restrict__ out,
-                                    int nh, int splits, int total_tokens, int first_token) {
+                                    int nh, int splits, int total_tokens, int first_token, const float* __restrict__ sinks) {
   const size_t token = (size_t)blockIdx.x + first_token;  // (the launch covers tokens [first_token, total_tokens))
   const int head = blockIdx.y;
   const size_t stride = (size_t)total_tokens * nh;  // slots per split
@@ -1293,8 +1302,9 @@ __global__ void merge_splits_kernel(const float* __restrict__ part_o, const floa
 #pragma unroll 8
   for (int s = 0; s < splits; ++s) mx = fmaxf(mx, part_lse[s * stride + slot0]);
   const float m_safe = (mx == -INFINITY) ? 0.f : mx;
+  const float sink_term = (sinks != nullptr && mx != -INFINITY) ? expf(sinks[head] - m_safe) : 0.f;
   for (int dd = threadIdx.x; dd < D; dd += blockDim.x) {
-    float acc = 0.f, denom = 0.f;
+    float acc = 0.f, denom = sink_term;
 #pragma unroll 8
     for (int s = 0; s < splits; ++s) {
       const size_t slot = s * stride + slot0;
@@ -1329,7 +1339,7 @@ template <typename T>
 static int launch(const void* qkv, int qkv_stride, const void* k_cache, const void* v_cache, const int* block_tables, int table_width,
                   const int* cu_q, const int* kv_lens, void* out, float* part_o, float* part_lse, int num_seqs, int total_tokens,
                   int max_q_len, int max_kv_len, int nh, int nkv, int page_shift, float scale, int window, int splits, int first_token,
-                  const float* bias_table, int bias_len, hipStream_t stream) {
+                  const float* bias_table, int bias_len, const float* sinks, hipStream_t stream) {
   constexpr int BN = tile_keys<T>();
   const int group = nh / nkv;
   // the streaming kernel keeps the page ids of a split's keys in LDS: they have to fit
@@ -1342,10 +1352,10 @@ static int launch(const void* qkv, int qkv_stride, const void* k_cache, const vo
     constexpr int DEPTH = sizeof(T) * D <= 256 ? 3 : 2;
     decode_attention_kernel<T, DEPTH, 4><<<dim3(splits, nkv, num_seqs), 256, 0, stream>>>(
         (const T*)qkv, qkv_stride, (const T*)k_cache, (const T*)v_cache, block_tables, table_width, kv_lens, (T*)out, part_o, part_lse,
-        nh, nkv, page_shift, scale, window, splits, total_tokens, bias_table, bias_len);
+        nh, nkv, page_shift, scale, window, splits, total_tokens, bias_table, bias_len, sinks);
     int status = (int)hipGetLastError();
     if (status != 0 || splits == 1) return status;
-    merge_splits_kernel<T><<<dim3(total_tokens, nh), D < 64 ? 64 : D, 0, stream>>>(part_o, part_lse, (T*)out, nh, splits, total_tokens, 0);
+    merge_splits_kernel<T><<<dim3(total_tokens, nh), D < 64 ? 64 : D, 0, stream>>>(part_o, part_lse, (T*)out, nh, splits, total_tokens, 0, sinks);
     return (int)hipGetLastError();
   }
   // The kernel whose tiles reach LDS by direct loads: bfloat16, head sizes 64 and 128, pages of at least 8 tokens.
@@ -1358,16 +1368,16 @@ static int launch(const void* qkv, int qkv_stride, const void* k_cache, const vo
       if (two_sets)
         direct_attention_kernel<2, 4, 2><<<grid, 512, 0, stream>>>(
             (const bf16_t*)qkv, qkv_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables, table_width, cu_q, kv_lens, (bf16_t*)out,
-            part_o, part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens, bias_table, bias_len);
+            part_o, part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens, bias_table, bias_len, sinks);
       else
         direct_attention_kernel<2, 4><<<grid, 256, 0, stream>>>(
             (const bf16_t*)qkv, qkv_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables, table_width, cu_q, kv_lens, (bf16_t*)out,
-            part_o, part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens, bias_table, bias_len);
+            part_o, part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens, bias_table, bias_len, sinks);
     }
     int status = (int)hipGetLastError();
     if (status != 0 || splits == 1) return status;
     merge_splits_kernel<T><<<dim3(total_tokens - first_token, nh), D < 64 ? 64 : D, 0, stream>>>(part_o, part_lse, (T*)out, nh, splits, total_tokens,
-                                                                                                 first_token);
+                                                                                                 first_token, sinks);
     return (int)hipGetLastError();
   };
   if (direct_ok && portion_kernel_choice >= 2 && max_q_len * group > 64) return launch_direct(portion_kernel_choice == 3);
@@ -1420,34 +1430,34 @@ static int launch(const void* qkv, int qkv_stride, const void* k_cache, const vo
       if (rows >= 256 && workgroups * 4 >= 7LL * compute_units()) {
         paged_attention_kernel<T, BN, 2, 1, 4><<<grid, 256, 0, stream>>>(
             (const T*)qkv, qkv_stride, (const T*)k_cache, (const T*)v_cache, block_tables, table_width, cu_q, kv_lens, (T*)out, part_o,
-            part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens, bias_table, bias_len);
+            part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens, bias_table, bias_len, sinks);
       } else {
         paged_attention_kernel<T, BN, 1, 1, 8><<<grid, 512, 0, stream>>>(
             (const T*)qkv, qkv_stride, (const T*)k_cache, (const T*)v_cache, block_tables, table_width, cu_q, kv_lens, (T*)out, part_o,
-            part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens, bias_table, bias_len);
+            part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens, bias_table, bias_len, sinks);
       }
     } else {
       dim3 grid(num_seqs * splits, nkv, (rows + 255) / 256);
       paged_attention_kernel<T, BN, WIDE, 1, 8><<<grid, 512, 0, stream>>>(
           (const T*)qkv, qkv_stride, (const T*)k_cache, (const T*)v_cache, block_tables, table_width, cu_q, kv_lens, (T*)out, part_o,
-          part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens, bias_table, bias_len);
+          part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens, bias_table, bias_len, sinks);
     }
   } else if (WIDE == 2 && (long long)((rows + 63) / 64) * nkv * num_seqs * splits < 2 * compute_units() && max_kv_len >= 8 * BN) {
     // too few workgroups to fill the GPU and many keys each: two sets of waves share a workgroup's keys
     dim3 grid(num_seqs * splits, nkv, (rows + 63) / 64);
     paged_attention_kernel<T, BN, 1, WIDE><<<grid, 256 * WIDE, 0, stream>>>(
         (const T*)qkv, qkv_stride, (const T*)k_cache, (const T*)v_cache, block_tables, table_width, cu_q, kv_lens, (T*)out, part_o,
-        part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens, bias_table, bias_len);
+        part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens, bias_table, bias_len, sinks);
   } else {
     dim3 grid(num_seqs * splits, nkv, (rows + 63) / 64);
     paged_attention_kernel<T, BN, 1, 1><<<grid, 256, 0, stream>>>(
         (const T*)qkv, qkv_stride, (const T*)k_cache, (const T*)v_cache, block_tables, table_width, cu_q, kv_lens, (T*)out, part_o,
-        part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens, bias_table, bias_len);
+        part_lse, nh, nkv, page_shift, scale, window, splits, total_tokens, bias_table, bias_len, sinks);
   }
   int status = (int)hipGetLastError();
   if (status != 0 || splits == 1) return status;
   merge_splits_kernel<T><<<dim3(total_tokens - first_token, nh), D < 64 ? 64 : D, 0, stream>>>(part_o, part_lse, (T*)out, nh, splits, total_tokens,
-                                                                                               first_token);
+                                                                                               first_token, sinks);
   return (int)hipGetLastError();
 }
 
@@ -1461,13 +1471,14 @@ extern "C" int velox_paged_attention(const void* qkv, int qkv_stride, const void
                                      const int* block_tables, int table_width, const int* cu_q, const int* kv_lens, void* out,
                                      float* part_o, float* part_lse, int num_seqs, int total_tokens, int max_q_len, int max_kv_len,
                                      int nh, int nkv, int page_shift, float scale, int window, int splits, int first_token, int dtype,
-                                     const float* bias_table, int bias_len, hipStream_t stream) {
+                                     const float* bias_table, int bias_len, const float* sinks, hipStream_t stream) {
+  // sinks: float32 [nh] or nullptr; exp(sinks[h]) joins the softmax's denominator of every row of head h (no key, no value, not scaled)
   if (num_seqs <= 0 || total_tokens <= 0) return 0;
   if (BIASED ? (bias_table == nullptr || bias_len < 1) : bias_table != nullptr) return -1;  // (the build and the call must agree)
   if (nh % nkv != 0 || splits < 1 || page_shift < 0 || max_kv_len < 1 || first_token < 0 || first_token >= total_tokens) return -1;
   if (dtype == VELOX_BF16)
     return launch<bf16_t>(qkv, qkv_stride, k_cache, v_cache, block_tables, table_width, cu_q, kv_lens, out, part_o, part_lse, num_seqs,
-                          total_tokens, max_q_len, max_kv_len, nh, nkv, page_shift, scale, window, splits, first_token, bias_table, bias_len, stream);
+                          total_tokens, max_q_len, max_kv_len, nh, nkv, page_shift, scale, window, splits, first_token, bias_table, bias_len, sinks, stream);
   return launch<float>(qkv, qkv_stride, k_cache, v_cache, block_tables, table_width, cu_q, kv_lens, out, part_o, part_lse, num_seqs,
-                       total_tokens, max_q_len, max_kv_len, nh, nkv, page_shift, scale, window, splits, first_token, bias_table, bias_len, stream);
+                       total_tokens, max_q_len, max_kv_len, nh, nkv, page_shift, scale, window, splits, first_token, bias_table, bias_len, sinks, stream);
 }

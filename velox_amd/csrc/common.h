@@ -102,4 +102,11 @@ __device__ __forceinline__ float glu_middle(float gate, float up, const GluUnit&
   return g / (1.f + expf(-unit.alpha * g)) * (u + unit.shift);
 }
 
+// The middle of a unit without a gate branch, act(up): kind 1 is relu(up)^2 (any other kind passes the value).
+#define VELOX_ACT_RELU2 1
+__device__ __forceinline__ float ungated_act(float v, int kind) {
+  const float r = fmaxf(v, 0.f);
+  return kind == VELOX_ACT_RELU2 ? r * r : v;
+}
+
 #define VELOX_RETURN_LAUNCH_STATUS() return (int)hipGetLastError()

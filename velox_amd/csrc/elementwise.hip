@@ -549,3 +549,191 @@ extern "C" int velox_row_scale_apply(const void* x, const float* sums, int block
   row_scale_apply_kernel<<<m, 256, 0, stream>>>((const bf16_t*)x, sums, blocks, inv_width, eps, (bf16_t*)out, n);
   VELOX_RETURN_LAUNCH_STATUS();
 }
+
+// ---------------------------------------------------------------------------------------------
+// embedding with a hashed table of token pairs:
+//   out[t, :] = float(table[ids[t], :]) * scale + float(bigram[row(t), :])
+//   row(t) = buckets                                                  at position 0
+//          = (previous * mul_prev + ids[t] * mul_cur) mod buckets     otherwise (64-bit arithmetic)
+// `previous` is ids[t - 1] inside a sequence's portion and, for a portion's first token, what the sequence's state
+// holds (state[slots[b]]); the workgroup that works a portion's first token reads the state and THEN sets it to the
+// portion's last token, so no other workgroup touches the entry.  Grid: (row blocks of a sequence, sequences); an id
+// outside the table yields NaN rows.
+// ---------------------------------------------------------------------------------------------
+template <typename T>
+__global__ void __launch_bounds__(256) embed_bigram_kernel(const int* __restrict__ ids, const T* __restrict__ table, const T* __restrict__ bigram,
+                                                           float* __restrict__ out, int hidden, int vocab, float scale, long long buckets,
+                                                           long long mul_prev, long long mul_cur, const int* __restrict__ positions,
+                                                           const int* __restrict__ cu_q, const int* __restrict__ slots, int* __restrict__ state) {
+  const int b = blockIdx.y;
+  const int first = cu_q[b], last = cu_q[b + 1] - 1;
+  const int t = first + blockIdx.x;
+  if (t > last) return;  // (uniform over the workgroup)
+  const int id = ids[t];
+  int previous = 0;
+  if (t == first) {
+    int* mine = state + slots[b];
+    previous = *mine;
+    __syncthreads();  // (every thread has read the entry before one of them overwrites it)
+    if (threadIdx.x == 0) *mine = ids[last];
+  } else {
+    previous = ids[t - 1];
+  }
+  float* dst = out + (size_t)t * hidden;
+  if (id < 0 || id >= vocab) {
+    for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = __builtin_nanf("");
+    return;
+  }
+  const long long row = positions[t] == 0 ? buckets : ((long long)previous * mul_prev + (long long)id * mul_cur) % buckets;
+  const T* src = table + (size_t)id * hidden;
+  const T* pair = bigram + (size_t)row * hidden;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = to_f32(src[i]) * scale + to_f32(pair[i]);
+}
+
+extern "C" int velox_embed_bigram(const int* ids, const void* table, const void* bigram, float* out, int tokens, int num_seqs, int max_q_len, int hidden,
+                                  int vocab, int table_dtype, float scale, int buckets, int mul_prev, int mul_cur, const int* positions, const int* cu_q,
+                                  const int* slots, int* state, hipStream_t stream) {
+  if (tokens <= 0 || num_seqs <= 0) return 0;
+  if (buckets < 1 || mul_prev < 0 || mul_cur < 0 || max_q_len < 1 || num_seqs > 65535) return -1;
+  dim3 grid(max_q_len, num_seqs);
+  if (table_dtype == VELOX_BF16)
+    embed_bigram_kernel<bf16_t><<<grid, 256, 0, stream>>>(ids, (const bf16_t*)table, (const bf16_t*)bigram, out, hidden, vocab, scale, buckets, mul_prev,
+                                                          mul_cur, positions, cu_q, slots, state);
+  else
+    embed_bigram_kernel<float><<<grid, 256, 0, stream>>>(ids, (const float*)table, (const float*)bigram, out, hidden, vocab, scale, buckets, mul_prev, mul_cur,
+                                                         positions, cu_q, slots, state);
+  VELOX_RETURN_LAUNCH_STATUS();
+}
+
+// ---------------------------------------------------------------------------------------------
+// residual add + a norm without statistics (Dynamic Tanh).  One block per output row, 16-byte accesses when the row
+// allows them.
+//   rows == nullptr: r = residual[row] (+ delta[row]); residual[row] = r; out[row] = tanh(alpha r) * w + b
+//   rows != nullptr: r = residual[rows[row]] (+ delta[rows[row]]); out[row] = the same; nothing else is written
+// delta may be `partials` stacked tensors `partial_stride` elements apart (added first to last), and with `second` the
+// delta is (p0 + p1 + ..) + second, as for add_rmsnorm.  alpha is read from device memory (one float).
+// ---------------------------------------------------------------------------------------------
+template <typename TD, typename TO>
+__global__ void __launch_bounds__(256) add_dynamic_tanh_kernel(float* __restrict__ residual, const TD* __restrict__ delta, const int* __restrict__ rows,
+                                                               const float* __restrict__ weight, const float* __restrict__ bias,
+                                                               const float* __restrict__ alpha_at, TO* __restrict__ out, int hidden, int partials,
+                                                               size_t partial_stride, const void* __restrict__ second, int second_bf16, int vec) {
+  const int row = blockIdx.x;
+  const size_t src_row = rows ? (size_t)rows[row] : (size_t)row;
+  float* res = residual + src_row * hidden;
+  const TD* del = delta ? delta + src_row * hidden : nullptr;
+  const bool write_back = (rows == nullptr) && (delta != nullptr);
+  const float alpha = *alpha_at;
+  TO* dst = out + (size_t)row * hidden;
+  if (vec) {
+    for (int at = 4 * threadIdx.x; at < hidden; at += 4 * blockDim.x) {
+      float4_t r = *reinterpret_cast<const float4_t*>(res + at);
+      if (del) {
+        float4_t d = {0.f, 0.f, 0.f, 0.f};
+        for (int p = 0; p < partials; ++p) {
+          Quad<TD> q;
+          q.v = *reinterpret_cast<const decltype(q.v)*>(del + p * partial_stride + at);
+#pragma unroll
+          for (int j = 0; j < 4; ++j) d[j] += q.get(j);
+        }
+        if (second) {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) d[j] += second_at(second, second_bf16, src_row * hidden + at + j);
+        }
+        r += d;
+        if (write_back) *reinterpret_cast<float4_t*>(res + at) = r;
+      }
+      const float4_t w = *reinterpret_cast<const float4_t*>(weight + at);
+      const float4_t bv = *reinterpret_cast<const float4_t*>(bias + at);
+      Quad<TO> o;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) o.set(j, tanhf(alpha * r[j]) * w[j] + bv[j]);
+      *reinterpret_cast<decltype(o.v)*>(dst + at) = o.v;
+    }
+    return;
+  }
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    float r = res[i];
+    if (del) {
+      float d = 0.f;
+      for (int p = 0; p < partials; ++p) d += to_f32(del[p * partial_stride + i]);
+      if (second) d += second_at(second, second_bf16, src_row * hidden + i);
+      r += d;
+      if (write_back) res[i] = r;
+    }
+    dst[i] = from_f32<TO>(tanhf(alpha * r) * weight[i] + bias[i]);
+  }
+}
+
+extern "C" int velox_add_dynamic_tanh(float* residual, const void* delta, const int* rows, const float* weight, const float* bias, const float* alpha,
+                                      void* out, int num_rows, int hidden, int delta_dtype, int out_dtype, int partials, long long partial_stride,
+                                      const void* second, int second_bf16, hipStream_t stream) {
+  if (num_rows <= 0) return 0;
+  if (hidden < 1 || partials < 1 || alpha == nullptr) return -1;
+  const int vec = hidden % 4 == 0 && (((uintptr_t)residual | (uintptr_t)delta | (uintptr_t)out | (uintptr_t)weight | (uintptr_t)bias) & 15) == 0 &&
+                  (partial_stride % 4 == 0);
+  const int threads = hidden >= 1024 ? 256 : (hidden >= 256 ? 64 * ((hidden / 4 + 63) / 64) : 64);
+#define VELOX_DYT(TD, TO)                                                                                                                         \
+  add_dynamic_tanh_kernel<TD, TO><<<num_rows, threads, 0, stream>>>(residual, (const TD*)delta, rows, weight, bias, alpha, (TO*)out, hidden, partials, \
+                                                                   (size_t)partial_stride, second, second_bf16, vec)
+  if (delta_dtype == VELOX_BF16 && out_dtype == VELOX_BF16) VELOX_DYT(bf16_t, bf16_t);
+  else if (delta_dtype == VELOX_F32 && out_dtype == VELOX_BF16) VELOX_DYT(float, bf16_t);
+  else if (delta_dtype == VELOX_F32 && out_dtype == VELOX_F32) VELOX_DYT(float, float);
+  else return -1;
+#undef VELOX_DYT
+  VELOX_RETURN_LAUNCH_STATUS();
+}
+
+// x[i] *= factor, float32, in place.
+__global__ void __launch_bounds__(256) scale_kernel(float* __restrict__ x, long long n, float factor) {
+  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long long)gridDim.x * blockDim.x) x[i] *= factor;
+}
+
+extern "C" int velox_scale(float* x, long long n, float factor, hipStream_t stream) {
+  if (n <= 0) return 0;
+  long long blocks = (n + 255) / 256;
+  if (blocks > 4096) blocks = 4096;
+  scale_kernel<<<(int)blocks, 256, 0, stream>>>(x, n, factor);
+  VELOX_RETURN_LAUNCH_STATUS();
+}
+
+// out[i] = act(x[i]) for a unit without a gate branch (ungated_act in common.h).  float32 arithmetic, one rounding.
+
+template <typename T>
+__global__ void __launch_bounds__(256) activation_kernel(const T* __restrict__ x, T* __restrict__ out, long long n, int kind) {
+  for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long long)gridDim.x * blockDim.x)
+    out[i] = from_f32<T>(ungated_act(to_f32(x[i]), kind));
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256) activation_vec_kernel(const T* __restrict__ x, T* __restrict__ out, long long pieces, int kind) {
+  constexpr int N = 16 / sizeof(T);
+  for (long long p = (long long)blockIdx.x * blockDim.x + threadIdx.x; p < pieces; p += (long long)gridDim.x * blockDim.x) {
+    const float4_t in = *reinterpret_cast<const float4_t*>(x + p * N);
+    float4_t ov;
+    const T* ie = reinterpret_cast<const T*>(&in);
+    T* oe = reinterpret_cast<T*>(&ov);
+#pragma unroll
+    for (int j = 0; j < N; ++j) oe[j] = from_f32<T>(ungated_act(to_f32(ie[j]), kind));
+    *reinterpret_cast<float4_t*>(out + p * N) = ov;
+  }
+}
+
+extern "C" int velox_activation(const void* x, void* out, long long n, int kind, int dtype, hipStream_t stream) {
+  if (n <= 0) return 0;
+  if (kind != 1) return -1;
+  const int per = dtype == VELOX_BF16 ? 8 : 4;
+  if (n % per == 0 && (((uintptr_t)x | (uintptr_t)out) & 15) == 0) {
+    const long long pieces = n / per;
+    long long blocks = (pieces + 255) / 256;
+    if (blocks > 8192) blocks = 8192;
+    if (dtype == VELOX_BF16) activation_vec_kernel<bf16_t><<<(int)blocks, 256, 0, stream>>>((const bf16_t*)x, (bf16_t*)out, pieces, kind);
+    else activation_vec_kernel<float><<<(int)blocks, 256, 0, stream>>>((const float*)x, (float*)out, pieces, kind);
+    VELOX_RETURN_LAUNCH_STATUS();
+  }
+  long long blocks = (n + 255) / 256;
+  if (blocks > 8192) blocks = 8192;
+  if (dtype == VELOX_BF16) activation_kernel<bf16_t><<<(int)blocks, 256, 0, stream>>>((const bf16_t*)x, (bf16_t*)out, n, kind);
+  else activation_kernel<float><<<(int)blocks, 256, 0, stream>>>((const float*)x, (float*)out, n, kind);
+  VELOX_RETURN_LAUNCH_STATUS();
+}

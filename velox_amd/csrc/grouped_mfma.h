@@ -23,7 +23,7 @@ typedef __bf16 gm_bf16x8_t __attribute__((ext_vector_type(8)));
 #define GM_ROWS 64       // rows of a tile without a plan (a plan's tiles hold 64 or 128)
 #define GM_FEW_COLS 32   // output columns of a workgroup of the kernel for few rows (GLU: 16)
 
-enum { GM_PLAIN = 0, GM_GLU = 1, GM_GATE = 2, GM_ROW_SCALE = 3 };
+enum { GM_PLAIN = 0, GM_GLU = 1, GM_GATE = 2, GM_ROW_SCALE = 3, GM_ACT = 4 };
 
 struct GroupedArgs {
   const bf16_t* a;     // element (row r, group g, k) at a[r * a_ld + g * a_group + k]
@@ -38,8 +38,9 @@ struct GroupedArgs {
   int m;
   const int* plan;
   int plan_pairs, plan_groups, plan_max_tiles;
-  const bf16_t* gate;  // GM_GATE: times sigmoid(gate[r * gate_ld + g * n + col])
-  long long gate_ld;
+  const bf16_t* gate;  // GM_GATE: times sigmoid(gate[r * gate_ld + g * gate_group + col * gate_col]); (n, 1) is a number per output, (1, 0) one per group
+  long long gate_ld, gate_group, gate_col;
+  int act = 0;         // GM_ACT: the result goes through ungated_act(., act)
   const float* row_scale;  // GM_ROW_SCALE: times row_scale[order[r]]
   GluUnit unit = {1.f, INFINITY, 0.f};  // GM_GLU: the unit's middle (see glu_middle)
 };
@@ -174,10 +175,11 @@ __global__ void __launch_bounds__(256) grouped_mfma_kernel(const GroupedArgs arg
         float v = acc[t][mt][j];
         if (EPI == GM_GLU) v = glu_middle(v, acc[t + GM_NT / 2][mt][j], args.unit);
         if (EPI == GM_GATE) {
-          const float z = to_f32(args.gate[(size_t)(row0 + r) * args.gate_ld + (size_t)group * n + col]);
+          const float z = to_f32(args.gate[(size_t)(row0 + r) * args.gate_ld + (size_t)group * args.gate_group + (size_t)col * args.gate_col]);
           v *= 1.f / (1.f + expf(-z));
         }
         if (EPI == GM_ROW_SCALE) v *= scale;
+        if (EPI == GM_ACT) v = ungated_act(v, args.act);
         out[out_row + col] = from_f32<TO>(v);
       }
   }
@@ -282,10 +284,11 @@ __global__ void __launch_bounds__(256) grouped_mfma_few_rows_kernel(const Groupe
         float v = acc[t][mt][j];
         if (EPI == GM_GLU) v = glu_middle(v, acc[1][mt][j], args.unit);
         if (EPI == GM_GATE) {
-          const float z = to_f32(args.gate[(size_t)(row0 + r) * args.gate_ld + (size_t)group * n + col]);
+          const float z = to_f32(args.gate[(size_t)(row0 + r) * args.gate_ld + (size_t)group * args.gate_group + (size_t)col * args.gate_col]);
           v *= 1.f / (1.f + expf(-z));
         }
         if (EPI == GM_ROW_SCALE) v *= scale;
+        if (EPI == GM_ACT) v = ungated_act(v, args.act);
         out[out_row + col] = from_f32<TO>(v);
       }
   }

@@ -40,10 +40,22 @@ __global__ void __launch_bounds__(256) latent_rotate_write_kernel(const T* __res
                                                                   const float* __restrict__ cos_table, const float* __restrict__ sin_table, int half,
                                                                   int interleaved, const float* __restrict__ norm_weight, float eps,
                                                                   const int* __restrict__ slots, T* __restrict__ k_cache, T* __restrict__ v_cache,
-                                                                  int page_size) {
+                                                                  int page_size, int norm2_offset, int norm2_size, const float* __restrict__ norm2_weight,
+                                                                  T* __restrict__ norm2_out) {
   __shared__ float scratch[16];
   const int t = blockIdx.x;
   const T* row = projected + (size_t)t * width;
+  if (norm2_out != nullptr) {  // (uniform) a second slice of the row, RMS-normed with its own weight: the queries' latent
+    const T* part = row + norm2_offset;
+    float sq = 0.f;
+    for (int i = threadIdx.x; i < norm2_size; i += blockDim.x) {
+      const float x = to_f32(part[i]);
+      sq += x * x;
+    }
+    const float inv2 = 1.0f / sqrtf(block_sum(sq, scratch) / (float)norm2_size + eps);
+    T* dst = norm2_out + (size_t)t * norm2_size;
+    for (int i = threadIdx.x; i < norm2_size; i += blockDim.x) dst[i] = from_f32<T>(to_f32(part[i]) * inv2 * norm2_weight[i]);
+  }
   const int pos = positions[t];
   const float* cs = half ? cos_table + (size_t)pos * half : nullptr;
   const float* sn = half ? sin_table + (size_t)pos * half : nullptr;
@@ -81,18 +93,22 @@ __global__ void __launch_bounds__(256) latent_rotate_write_kernel(const T* __res
 extern "C" int velox_latent_rotate_write(const void* projected, int width, void* queries, int tokens, int heads, int dim, int rot, int rank, int cached,
                                          int down_offset, const int* positions, const float* cos_table, const float* sin_table, int half, int interleaved,
                                          const float* norm_weight, float eps, const int* slots, void* k_cache, void* v_cache, int page_size, int dtype,
-                                         hipStream_t stream) {
+                                         int norm2_offset, int norm2_size, const float* norm2_weight, void* norm2_out, hipStream_t stream) {
   if (tokens <= 0) return 0;
-  if (heads < 1 || dim < 1 || rot < 0 || rank < 1 || cached < rank + rot || 2 * half > rot || page_size < 1) return -1;
+  // (heads == 0: no queries, only the cache write and the second norm)
+  if (heads < 0 || dim < 0 || (heads > 0 && dim < 1) || rot < 0 || rank < 1 || cached < rank + rot || 2 * half > rot || page_size < 1) return -1;
   if (heads * (dim + rot) > width || (down_offset >= 0 && (down_offset + rank + rot > width || norm_weight == nullptr))) return -1;
+  if (norm2_out != nullptr && (norm2_offset < 0 || norm2_size < 1 || norm2_offset + norm2_size > width || norm2_weight == nullptr)) return -1;
   if (dtype == VELOX_BF16)
     latent_rotate_write_kernel<bf16_t><<<tokens, 256, 0, stream>>>((const bf16_t*)projected, width, (bf16_t*)queries, heads, dim, rot, rank, cached, down_offset,
                                                                    positions, cos_table, sin_table, half, interleaved, norm_weight, eps, slots,
-                                                                   (bf16_t*)k_cache, (bf16_t*)v_cache, page_size);
+                                                                   (bf16_t*)k_cache, (bf16_t*)v_cache, page_size, norm2_offset, norm2_size, norm2_weight,
+                                                                   (bf16_t*)norm2_out);
   else
     latent_rotate_write_kernel<float><<<tokens, 256, 0, stream>>>((const float*)projected, width, (float*)queries, heads, dim, rot, rank, cached, down_offset,
                                                                   positions, cos_table, sin_table, half, interleaved, norm_weight, eps, slots,
-                                                                  (float*)k_cache, (float*)v_cache, page_size);
+                                                                  (float*)k_cache, (float*)v_cache, page_size, norm2_offset, norm2_size, norm2_weight,
+                                                                  (float*)norm2_out);
   VELOX_RETURN_LAUNCH_STATUS();
 }
 
@@ -114,7 +130,7 @@ template <typename T>
 __global__ void __launch_bounds__(256) head_linear_kernel(const T* __restrict__ x, int x_width, int x_stride, int x_offset, const T* __restrict__ maps,
                                                           T* __restrict__ out, int out_width, int out_stride, int out_offset,
                                                           const T* __restrict__ gate, int gate_width, int gate_offset, int m, int n, int k,
-                                                          int x_vec, int w_vec) {
+                                                          int x_vec, int w_vec, int gate_per_head) {
   __shared__ float a_tile[HL_BK][HL_BM + HL_PAD];
   __shared__ float w_tile[HL_BK][HL_BN + HL_PAD];
   const int g = blockIdx.z;
@@ -171,7 +187,7 @@ __global__ void __launch_bounds__(256) head_linear_kernel(const T* __restrict__ 
       if (col >= n) continue;
       float v = total[i][j] + acc[i][j];
       if (gate) {
-        const float z = to_f32(gate[(size_t)row * gate_width + gate_offset + g * n + col]);
+        const float z = to_f32(gate[(size_t)row * gate_width + gate_offset + (gate_per_head ? g : g * n + col)]);
         v *= 1.f / (1.f + expf(-z));
       }
       out[(size_t)row * out_width + (size_t)g * out_stride + out_offset + col] = from_f32<T>(v);
@@ -181,10 +197,11 @@ __global__ void __launch_bounds__(256) head_linear_kernel(const T* __restrict__ 
 
 extern "C" int velox_head_linear(const void* x, int x_width, int x_stride, int x_offset, const void* maps, void* out, int out_width, int out_stride,
                                  int out_offset, const void* gate, int gate_width, int gate_offset, int m, int groups, int n, int k, int dtype,
-                                 hipStream_t stream) {
+                                 int gate_per_head, hipStream_t stream) {
   if (m <= 0 || groups <= 0 || n <= 0) return 0;
   if (k < 1 || groups > 65535 || (groups - 1) * x_stride + x_offset + k > x_width || (groups - 1) * out_stride + out_offset + n > out_width) return -1;
-  if (gate != nullptr && gate_offset + groups * n > gate_width) return -1;
+  // (gate_per_head: the gate holds one number per group, times every output of the group)
+  if (gate != nullptr && gate_offset + (gate_per_head ? groups : groups * n) > gate_width) return -1;
   if (dtype == VELOX_BF16 && grouped_mfma_fits(x, x_width, x_stride, x_offset, maps, k)) {
     // bfloat16: the same sums on the matrix cores
     GroupedArgs args = {};
@@ -201,6 +218,8 @@ extern "C" int velox_head_linear(const void* x, int x_width, int x_stride, int x
     args.m = m;
     args.gate = gate ? (const bf16_t*)gate + gate_offset : nullptr;
     args.gate_ld = gate_width;
+    args.gate_group = gate_per_head ? 1 : n;
+    args.gate_col = gate_per_head ? 0 : 1;
     const int row_tiles = (m + GM_ROWS - 1) / GM_ROWS;
     if (row_tiles > 65535) return -1;
     if (gate) grouped_mfma_launch<GM_GATE, bf16_t>(args, m, GM_ROWS, row_tiles, groups, stream);
@@ -214,10 +233,10 @@ extern "C" int velox_head_linear(const void* x, int x_width, int x_stride, int x
   const int w_vec = k % 4 == 0 && ((uintptr_t)maps) % (4 * size) == 0;
   if (dtype == VELOX_BF16)
     head_linear_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)x, x_width, x_stride, x_offset, (const bf16_t*)maps, (bf16_t*)out, out_width, out_stride,
-                                                         out_offset, (const bf16_t*)gate, gate_width, gate_offset, m, n, k, x_vec, w_vec);
+                                                         out_offset, (const bf16_t*)gate, gate_width, gate_offset, m, n, k, x_vec, w_vec, gate_per_head);
   else
     head_linear_kernel<float><<<grid, 256, 0, stream>>>((const float*)x, x_width, x_stride, x_offset, (const float*)maps, (float*)out, out_width, out_stride,
-                                                        out_offset, (const float*)gate, gate_width, gate_offset, m, n, k, x_vec, w_vec);
+                                                        out_offset, (const float*)gate, gate_width, gate_offset, m, n, k, x_vec, w_vec, gate_per_head);
   VELOX_RETURN_LAUNCH_STATUS();
 }
 
@@ -243,7 +262,8 @@ template <typename T>
 __global__ void __launch_bounds__(256) plain_attention_kernel(const T* __restrict__ q, int q_width, const T* __restrict__ k_cache, const T* __restrict__ v_cache,
                                                               const int* __restrict__ block_tables, int table_width, const int* __restrict__ cu_q,
                                                               const int* __restrict__ kv_lens, T* __restrict__ out, int num_seqs, int nh, int nkv, int d,
-                                                              int page_shift, float scale, int window, const float* __restrict__ bias_table, int bias_len) {
+                                                              int page_shift, float scale, int window, const float* __restrict__ bias_table, int bias_len,
+                                                              const float* __restrict__ sinks) {
   __shared__ float q_s[PLAIN_ATTENTION_MAX_D];
   __shared__ float p_s[256];
   __shared__ float scratch[16];
@@ -299,6 +319,8 @@ __global__ void __launch_bounds__(256) plain_attention_kernel(const T* __restric
     }
     __syncthreads();  // (p_s is written again in the next round)
   }
+  // a sink: exp(sinks[head]) joins the denominator (it has no key and no value and is not scaled)
+  if (sinks) denom += expf(sinks[head] - running_max);
 #pragma unroll
   for (int u = 0; u < PLAIN_ATTENTION_MAX_D / 256; ++u) {
     const int c = tid + 256 * u;
@@ -308,16 +330,16 @@ __global__ void __launch_bounds__(256) plain_attention_kernel(const T* __restric
 
 extern "C" int velox_plain_attention(const void* q, int q_width, const void* k_cache, const void* v_cache, const int* block_tables, int table_width,
                                      const int* cu_q, const int* kv_lens, void* out, int num_seqs, int tokens, int nh, int nkv, int d, int page_shift,
-                                     float scale, int window, int dtype, const float* bias_table, int bias_len, hipStream_t stream) {
+                                     float scale, int window, int dtype, const float* bias_table, int bias_len, const float* sinks, hipStream_t stream) {
   if (tokens <= 0) return 0;
   if (bias_table != nullptr && bias_len < 1) return -1;
   if (d < 1 || d > PLAIN_ATTENTION_MAX_D || nh < 1 || nkv < 1 || nh % nkv != 0 || nh > 65535 || num_seqs < 1 || nh * d > q_width) return -1;
   dim3 grid(tokens, nh);
   if (dtype == VELOX_BF16)
     plain_attention_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)q, q_width, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_tables, table_width,
-                                                             cu_q, kv_lens, (bf16_t*)out, num_seqs, nh, nkv, d, page_shift, scale, window, bias_table, bias_len);
+                                                             cu_q, kv_lens, (bf16_t*)out, num_seqs, nh, nkv, d, page_shift, scale, window, bias_table, bias_len, sinks);
   else
     plain_attention_kernel<float><<<grid, 256, 0, stream>>>((const float*)q, q_width, (const float*)k_cache, (const float*)v_cache, block_tables, table_width,
-                                                            cu_q, kv_lens, (float*)out, num_seqs, nh, nkv, d, page_shift, scale, window, bias_table, bias_len);
+                                                            cu_q, kv_lens, (float*)out, num_seqs, nh, nkv, d, page_shift, scale, window, bias_table, bias_len, sinks);
   VELOX_RETURN_LAUNCH_STATUS();
 }

@@ -370,7 +370,8 @@ extern "C" int velox_short_conv(const void* x, int ld, int channels, const float
 // ---------------------------------------------------------------------------------------------
 // rotate_pad_write: workgroups take a token's heads in turn (queries, keys, then values; one head each in steps of few tokens).  A row
 // of qkv holds `heads` queries and `kv_heads` keys of `dim` channels and `kv_heads` values of `vdim`.  The first 2 * half
-// channels of every query and key head are rotated (channel i with i + half, cos/sin float32 [positions, half]); queries go to
+// channels of every query and key head are rotated (channel i with i + half, or 2i with 2i + 1 when `interleaved`; cos/sin
+// float32 [positions, half]; (u, v) -> (u cos - v sin, v cos + u sin)); queries go to
 // q_out [T, heads * D], keys to k_cache [pages, kv_heads, page, D], values to v_cache [pages, kv_heads, D, page]; channels from
 // dim (vdim) to D are zeros.
 // ---------------------------------------------------------------------------------------------
@@ -378,7 +379,8 @@ template <typename T>
 __global__ void __launch_bounds__(256) rotate_pad_write_kernel(const T* __restrict__ qkv, int ld, T* __restrict__ q_out, const int* __restrict__ positions,
                                                                const float* __restrict__ cos_t, const float* __restrict__ sin_t, int half,
                                                                const int* __restrict__ slot_mapping, T* __restrict__ k_cache, T* __restrict__ v_cache,
-                                                               int heads, int kv_heads, int dim, int vdim, int D, int page_shift, int write_kv) {
+                                                               int heads, int kv_heads, int dim, int vdim, int D, int page_shift, int write_kv,
+                                                               int interleaved) {
   const int t = blockIdx.x;
   const T* row = qkv + (size_t)t * ld;
   const int q_size = heads * dim, k_size = kv_heads * dim;
@@ -408,7 +410,12 @@ __global__ void __launch_bounds__(256) rotate_pad_write_kernel(const T* __restri
       float v = 0.f;
       if (c < dim) {
         v = to_f32(src[c]);
-        if (c < half) v = v * cs[c] - to_f32(src[c + half]) * sn[c];
+        if (interleaved) {
+          if (c < 2 * half) {
+            const int i = c >> 1;
+            v = (c & 1) ? v * cs[i] + to_f32(src[c - 1]) * sn[i] : v * cs[i] - to_f32(src[c + 1]) * sn[i];
+          }
+        } else if (c < half) v = v * cs[c] - to_f32(src[c + half]) * sn[c];
         else if (c < 2 * half) v = v * cs[c - half] + to_f32(src[c - half]) * sn[c - half];
       }
       dst[c] = from_f32<T>(v);
@@ -418,7 +425,7 @@ __global__ void __launch_bounds__(256) rotate_pad_write_kernel(const T* __restri
 
 extern "C" int velox_rotate_pad_write(const void* qkv, int ld, void* q_out, const int* positions, const float* cos_t, const float* sin_t, int half,
                                       const int* slot_mapping, void* k_cache, void* v_cache, int tokens, int heads, int kv_heads, int dim, int vdim, int D,
-                                      int page_size, int write_kv, int dtype, hipStream_t stream) {
+                                      int page_size, int write_kv, int dtype, int interleaved, hipStream_t stream) {
   if (tokens <= 0) return 0;
   int shift = 0;
   while ((1 << shift) < page_size) ++shift;
@@ -429,10 +436,10 @@ extern "C" int velox_rotate_pad_write(const void* qkv, int ld, void* q_out, cons
   if (lanes > 256) lanes = 256;
   if (dtype == VELOX_BF16)
     rotate_pad_write_kernel<bf16_t><<<grid, lanes, 0, stream>>>((const bf16_t*)qkv, ld, (bf16_t*)q_out, positions, cos_t, sin_t, half, slot_mapping,
-                                                              (bf16_t*)k_cache, (bf16_t*)v_cache, heads, kv_heads, dim, vdim, D, shift, write_kv);
+                                                              (bf16_t*)k_cache, (bf16_t*)v_cache, heads, kv_heads, dim, vdim, D, shift, write_kv, interleaved);
   else
     rotate_pad_write_kernel<float><<<grid, lanes, 0, stream>>>((const float*)qkv, ld, (float*)q_out, positions, cos_t, sin_t, half, slot_mapping,
-                                                             (float*)k_cache, (float*)v_cache, heads, kv_heads, dim, vdim, D, shift, write_kv);
+                                                             (float*)k_cache, (float*)v_cache, heads, kv_heads, dim, vdim, D, shift, write_kv, interleaved);
   VELOX_RETURN_LAUNCH_STATUS();
 }
 

@@ -26,12 +26,16 @@
 // largest scores, ties to the lower index; weights are the chosen scores, divided by their sum when `renormalize`.
 // Every round the wave takes the largest score that is not yet taken (value first, then the lower index), so the choices
 // come out in descending order of score.  With `correction` (float32 [experts]) the choice goes by score + correction and
-// the weights stay the scores themselves.
+// the weights stay the scores themselves.  With `group_count` > 0 the experts form that many equal groups of neighbours; a
+// group's score is the sum of its two largest choice scores (of its one, if it has one expert), and only experts of the
+// `group_keep` best groups (ties to the lower index) can be chosen: the others' choice scores become minus infinity.
+// `norm_floor` is added to the sum that renormalised weights are divided by.
 // ---------------------------------------------------------------------------------------------
 #define ROUTE_PER_LANE 32  // experts per lane held in registers: up to 2,048 experts
 
 __global__ void __launch_bounds__(256) route_top_kernel(const float* __restrict__ logits, int* __restrict__ choice, float* __restrict__ weight, int tokens,
-                                                        int experts, int top, int softmax, int renormalize, const float* __restrict__ correction) {
+                                                        int experts, int top, int softmax, int renormalize, const float* __restrict__ correction,
+                                                        int group_count, int group_keep, float norm_floor) {
   const int lane = threadIdx.x & 63;
   const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (t >= tokens) return;  // (a whole wave; nothing below crosses waves)
@@ -53,6 +57,57 @@ __global__ void __launch_bounds__(256) route_top_kernel(const float* __restrict_
     if (e < experts) {
       score[u] = softmax ? expf(z[e] - shift) / denom : 1.f / (1.f + expf(-z[e]));
       if (correction) score[u] += correction[e];
+    }
+  }
+  if (group_count > 0) {
+    // lane g ends up with group g's score (group_count <= 64); every group's two largest by two rounds over the wave
+    const int per = experts / group_count;
+    float mine = -INFINITY;  // (lanes beyond the groups never win)
+    for (int gidx = 0; gidx < group_count; ++gidx) {
+      const int lo = gidx * per, hi = lo + per;
+      float first = -INFINITY, second = -INFINITY;  // this lane's two largest inside the group
+#pragma unroll
+      for (int u = 0; u < ROUTE_PER_LANE; ++u) {
+        const int e = lane + 64 * u;
+        if (e >= lo && e < hi) {
+          const float v = score[u];
+          if (v > first) { second = first; first = v; }
+          else if (v > second) second = v;
+        }
+      }
+      // the wave's two largest: merge (first, second) pairs
+#pragma unroll
+      for (int offset = 32; offset > 0; offset >>= 1) {
+        const float of = __shfl_xor(first, offset, 64), os = __shfl_xor(second, offset, 64);
+        const float hi1 = fmaxf(first, of);
+        const float lo1 = fminf(first, of);
+        second = fmaxf(lo1, fmaxf(second, os));
+        first = hi1;
+      }
+      const float sum = per > 1 ? first + second : first;
+      if (lane == gidx) mine = sum;
+    }
+    unsigned long long allowed = 0ull;
+    for (int k = 0; k < group_keep; ++k) {
+      float best = mine;
+      int best_g = lane < group_count ? lane : 0x7fffffff;
+      if (lane >= group_count || ((allowed >> lane) & 1ull)) { best = -INFINITY; best_g = 0x7fffffff; }
+#pragma unroll
+      for (int offset = 32; offset > 0; offset >>= 1) {
+        const float other = __shfl_xor(best, offset, 64);
+        const int other_g = __shfl_xor(best_g, offset, 64);
+        if (other > best || (other == best && other_g < best_g)) { best = other; best_g = other_g; }
+      }
+      if (best_g < group_count) allowed |= 1ull << best_g;
+      else {  // (every group left scores minus infinity or NaN: take the lowest group not yet taken)
+        for (int gidx = 0; gidx < group_count; ++gidx)
+          if (!((allowed >> gidx) & 1ull)) { allowed |= 1ull << gidx; break; }
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < ROUTE_PER_LANE; ++u) {
+      const int e = lane + 64 * u;
+      if (e < experts && !((allowed >> (e / per)) & 1ull)) score[u] = -INFINITY;
     }
   }
   float total = 0.f;
@@ -81,14 +136,18 @@ __global__ void __launch_bounds__(256) route_top_kernel(const float* __restrict_
     }
   }
   if (renormalize && lane == 0)  // (the lane that wrote them)
-    for (int k = 0; k < top; ++k) weight[(size_t)t * top + k] /= total;
+    for (int k = 0; k < top; ++k) weight[(size_t)t * top + k] /= (total + norm_floor);
 }
 
 extern "C" int velox_route_top(const float* logits, int* choice, float* weight, int tokens, int experts, int top, int softmax, int renormalize,
-                               const float* correction, hipStream_t stream) {
+                               const float* correction, int group_count, int group_keep, float norm_floor, hipStream_t stream) {
   if (tokens <= 0) return 0;
   if (experts < 1 || experts > 64 * ROUTE_PER_LANE || top < 1 || top > experts) return -1;
-  route_top_kernel<<<(tokens + 3) / 4, 256, 0, stream>>>(logits, choice, weight, tokens, experts, top, softmax, renormalize, correction);
+  if (group_count < 0 || group_count > 64 ||
+      (group_count > 0 && (experts % group_count != 0 || group_keep < 1 || group_keep > group_count || group_keep * (experts / group_count) < top)))
+    return -1;
+  route_top_kernel<<<(tokens + 3) / 4, 256, 0, stream>>>(logits, choice, weight, tokens, experts, top, softmax, renormalize, correction, group_count,
+                                                         group_keep, norm_floor);
   VELOX_RETURN_LAUNCH_STATUS();
 }
 
@@ -188,12 +247,16 @@ extern "C" int velox_routed_plan(const int* choice, int pairs, int experts, int*
 // ---------------------------------------------------------------------------------------------
 // The grouped products.  GLU: two tiles of W (gate rows and the up rows of the same columns), the activation as the
 // epilogue.  Rows of A: GLU gathers x[token] (scaled by the pair's weight and rounded to T, as a product on T operands
-// would read it); the down product reads the sorted rows of act.
+// would read it); the down product reads the sorted rows of act.  FIRST = 2: a unit without a gate branch, one tile of
+// W (the up rows), rows gathered as for GLU, ungated_act(., act_kind) as the epilogue.
 // ---------------------------------------------------------------------------------------------
-template <typename T, typename TO, bool GLU>
+template <typename T, typename TO, int FIRST>
 __global__ void __launch_bounds__(256) grouped_product_kernel(const T* __restrict__ a, const T* __restrict__ w, TO* __restrict__ out,
                                                               const int* __restrict__ plan, const float* __restrict__ pair_weight, int pairs, int experts,
-                                                              int max_tiles, int top, int n, int k, int scale_rows, int a_vec, int w_vec, GluUnit unit) {
+                                                              int max_tiles, int top, int n, int k, int scale_rows, int a_vec, int w_vec, GluUnit unit,
+                                                              int act_kind) {
+  constexpr bool GLU = FIRST == 1;       // two tiles of W and the gated epilogue
+  constexpr bool GATHERS = FIRST != 0;   // rows are x[token of the pair], not sorted rows
   __shared__ float a_tile[RT_BK][RT_BM + RT_PAD];
   __shared__ float w_tile[GLU ? 2 : 1][RT_BK][RT_BN + RT_PAD];
   __shared__ int row_pair[RT_BM];
@@ -217,7 +280,7 @@ __global__ void __launch_bounds__(256) grouped_product_kernel(const T* __restric
   size_t a_off = 0;
   float a_scale = 1.f;
   if (a_row_ok) {
-    if (GLU) {
+    if (GATHERS) {
       a_off = (size_t)(my_pair / top) * k;
       if (scale_rows) a_scale = pair_weight[my_pair];
     } else {
@@ -252,7 +315,7 @@ __global__ void __launch_bounds__(256) grouped_product_kernel(const T* __restric
     }
     float av[4], wv[NW][4];
     load4<T>(a, a_off, k0 + load_k, k, a_row_ok, a_vec != 0, av);
-    if (GLU && scale_rows) {
+    if (GATHERS && scale_rows) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) av[i] = to_f32(from_f32<T>(av[i] * a_scale));
     }
@@ -283,7 +346,7 @@ __global__ void __launch_bounds__(256) grouped_product_kernel(const T* __restric
   for (int i = 0; i < 4; ++i) {
     const int r = ty * 4 + i;
     if (r >= rows) continue;
-    const float row_scale = (!GLU && scale_rows) ? pair_weight[row_pair[r]] : 1.f;
+    const float row_scale = (!GATHERS && scale_rows) ? pair_weight[row_pair[r]] : 1.f;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int col = n0 + tx * 4 + j;
@@ -292,6 +355,8 @@ __global__ void __launch_bounds__(256) grouped_product_kernel(const T* __restric
       if (GLU) {
         const float up = total[NW - 1][i][j] + acc[NW - 1][i][j];
         v = glu_middle(v, up, unit);  // (float32 throughout, one rounding at the store)
+      } else if (FIRST == 2) {
+        v = ungated_act(v, act_kind);
       } else {
         v *= row_scale;
       }
@@ -301,7 +366,8 @@ __global__ void __launch_bounds__(256) grouped_product_kernel(const T* __restric
 }
 
 extern "C" int velox_grouped_glu(const void* x, const void* gate_up, void* act, const int* plan, const float* pair_weight, int pairs, int experts, int top,
-                                 int inter, int hidden, int scale_input, int dtype, float alpha, float limit, float shift, hipStream_t stream) {
+                                 int inter, int hidden, int scale_input, int dtype, float alpha, float limit, float shift, int ungated, hipStream_t stream) {
+  // `ungated` > 0: `gate_up` holds [experts * inter, hidden] (up rows only) and the unit is ungated_act(up, ungated)
   if (pairs <= 0) return 0;
   const GluUnit unit = {alpha, limit, shift};
   const int max_tiles = velox_routed_max_tiles(pairs, experts);
@@ -310,12 +376,21 @@ extern "C" int velox_grouped_glu(const void* x, const void* gate_up, void* act, 
   const int size = dtype == VELOX_BF16 ? 2 : 4;
   const int a_vec = hidden % 4 == 0 && ((uintptr_t)x) % (4 * size) == 0;
   const int w_vec = hidden % 4 == 0 && ((uintptr_t)gate_up) % (4 * size) == 0;
+  if (ungated > 0) {
+    if (dtype == VELOX_BF16)
+      grouped_product_kernel<bf16_t, bf16_t, 2><<<grid, 256, 0, stream>>>((const bf16_t*)x, (const bf16_t*)gate_up, (bf16_t*)act, plan, pair_weight, pairs, experts,
+                                                                          max_tiles, top, inter, hidden, scale_input, a_vec, w_vec, unit, ungated);
+    else
+      grouped_product_kernel<float, float, 2><<<grid, 256, 0, stream>>>((const float*)x, (const float*)gate_up, (float*)act, plan, pair_weight, pairs, experts,
+                                                                        max_tiles, top, inter, hidden, scale_input, a_vec, w_vec, unit, ungated);
+    VELOX_RETURN_LAUNCH_STATUS();
+  }
   if (dtype == VELOX_BF16)
-    grouped_product_kernel<bf16_t, bf16_t, true><<<grid, 256, 0, stream>>>((const bf16_t*)x, (const bf16_t*)gate_up, (bf16_t*)act, plan, pair_weight, pairs, experts,
-                                                                           max_tiles, top, inter, hidden, scale_input, a_vec, w_vec, unit);
+    grouped_product_kernel<bf16_t, bf16_t, 1><<<grid, 256, 0, stream>>>((const bf16_t*)x, (const bf16_t*)gate_up, (bf16_t*)act, plan, pair_weight, pairs, experts,
+                                                                        max_tiles, top, inter, hidden, scale_input, a_vec, w_vec, unit, 0);
   else
-    grouped_product_kernel<float, float, true><<<grid, 256, 0, stream>>>((const float*)x, (const float*)gate_up, (float*)act, plan, pair_weight, pairs, experts,
-                                                                         max_tiles, top, inter, hidden, scale_input, a_vec, w_vec, unit);
+    grouped_product_kernel<float, float, 1><<<grid, 256, 0, stream>>>((const float*)x, (const float*)gate_up, (float*)act, plan, pair_weight, pairs, experts,
+                                                                      max_tiles, top, inter, hidden, scale_input, a_vec, w_vec, unit, 0);
   VELOX_RETURN_LAUNCH_STATUS();
 }
 
@@ -329,11 +404,11 @@ extern "C" int velox_grouped_down(const void* act, const void* down, float* y, c
   const int a_vec = inter % 4 == 0 && ((uintptr_t)act) % (4 * size) == 0;
   const int w_vec = inter % 4 == 0 && ((uintptr_t)down) % (4 * size) == 0;
   if (dtype == VELOX_BF16)
-    grouped_product_kernel<bf16_t, float, false><<<grid, 256, 0, stream>>>((const bf16_t*)act, (const bf16_t*)down, y, plan, pair_weight, pairs, experts, max_tiles,
-                                                                           top, hidden, inter, scale_output, a_vec, w_vec, GluUnit{1.f, INFINITY, 0.f});
+    grouped_product_kernel<bf16_t, float, 0><<<grid, 256, 0, stream>>>((const bf16_t*)act, (const bf16_t*)down, y, plan, pair_weight, pairs, experts, max_tiles,
+                                                                       top, hidden, inter, scale_output, a_vec, w_vec, GluUnit{1.f, INFINITY, 0.f}, 0);
   else
-    grouped_product_kernel<float, float, false><<<grid, 256, 0, stream>>>((const float*)act, (const float*)down, y, plan, pair_weight, pairs, experts, max_tiles,
-                                                                          top, hidden, inter, scale_output, a_vec, w_vec, GluUnit{1.f, INFINITY, 0.f});
+    grouped_product_kernel<float, float, 0><<<grid, 256, 0, stream>>>((const float*)act, (const float*)down, y, plan, pair_weight, pairs, experts, max_tiles,
+                                                                      top, hidden, inter, scale_output, a_vec, w_vec, GluUnit{1.f, INFINITY, 0.f}, 0);
   VELOX_RETURN_LAUNCH_STATUS();
 }
 
@@ -373,7 +448,8 @@ static GroupedArgs routed_args(const void* a, const void* w, void* out, const in
 // inter % 8 == 0 (the caller checks).
 extern "C" int velox_routed_products_bf16(const void* x, const void* gate_up, const void* down, void* sorted, void* act, float* y, const int* plan,
                                           const float* pair_weight, int pairs, int experts, int top, int inter, int hidden, int scale_input,
-                                          int tile_rows, float alpha, float limit, float shift, hipStream_t stream) {
+                                          int tile_rows, float alpha, float limit, float shift, int ungated, hipStream_t stream) {
+  // `ungated` > 0: `gate_up` holds [experts * inter, hidden] (up rows only) and the unit is ungated_act(up, ungated)
   if (pairs <= 0) return 0;
   if (hidden % 8 != 0 || inter % 8 != 0) return -1;
   const int max_tiles = velox_routed_max_tiles(pairs, experts);
@@ -381,9 +457,15 @@ extern "C" int velox_routed_products_bf16(const void* x, const void* gate_up, co
   const int* order = plan + 1 + (experts + 1);
   if (x != nullptr)  // (nullptr: the plan kernel has copied the rows already)
     routed_gather_kernel<<<pairs, 256, 0, stream>>>((const bf16_t*)x, order, pair_weight, (bf16_t*)sorted, top, hidden, scale_input, plan + 1 + experts);
-  GroupedArgs glu = routed_args(sorted, gate_up, act, plan, pairs, experts, inter, hidden, 2 * inter);
-  glu.unit = GluUnit{alpha, limit, shift};
-  grouped_mfma_launch<GM_GLU, bf16_t>(glu, pairs, tile_rows, max_tiles, 1, stream);
+  if (ungated > 0) {
+    GroupedArgs first = routed_args(sorted, gate_up, act, plan, pairs, experts, inter, hidden, inter);
+    first.act = ungated;
+    grouped_mfma_launch<GM_ACT, bf16_t>(first, pairs, tile_rows, max_tiles, 1, stream);
+  } else {
+    GroupedArgs glu = routed_args(sorted, gate_up, act, plan, pairs, experts, inter, hidden, 2 * inter);
+    glu.unit = GluUnit{alpha, limit, shift};
+    grouped_mfma_launch<GM_GLU, bf16_t>(glu, pairs, tile_rows, max_tiles, 1, stream);
+  }
   GroupedArgs last = routed_args(act, down, y, plan, pairs, experts, hidden, inter, hidden);
   // (a weight on the experts' OUTPUT is applied where the results are added up, routed_combine with scale_rows: the product
   // itself is the same kernel either way)

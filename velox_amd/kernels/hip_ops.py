@@ -143,18 +143,18 @@ class HipOps:
         c.velox_probe_mfma.restype = _I
         c.velox_probe_grid_barrier.argtypes = [_I, _I, _I, _P, _P, _P]
         c.velox_probe_grid_barrier.restype = _I
-        c.velox_latent_rotate_write.argtypes = [_P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _P, _P, _P, _I, _I, _P, _F, _P, _P, _P, _I, _I, _P]
-        c.velox_head_linear.argtypes = [_P, _I, _I, _I, _P, _P, _I, _I, _I, _P, _I, _I, _I, _I, _I, _I, _I, _P]
-        c.velox_plain_attention.argtypes = [_P, _I, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _P, _I, _P]
+        c.velox_latent_rotate_write.argtypes = [_P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _P, _P, _P, _I, _I, _P, _F, _P, _P, _P, _I, _I, _I, _I, _P, _P, _P]
+        c.velox_head_linear.argtypes = [_P, _I, _I, _I, _P, _P, _I, _I, _I, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P]
+        c.velox_plain_attention.argtypes = [_P, _I, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _P, _I, _P, _P]
         c.velox_plain_attention.restype = _I
-        c.velox_route_top.argtypes = [_P, _P, _P, _I, _I, _I, _I, _I, _P, _P]
+        c.velox_route_top.argtypes = [_P, _P, _P, _I, _I, _I, _I, _I, _P, _I, _I, _F, _P]
         c.velox_routed_plan_elems.argtypes = [_I, _I]
         c.velox_routed_plan_elems.restype = ctypes.c_longlong
         c.velox_routed_plan.argtypes = [_P, _I, _I, _P, _I, _P, _P, _P, _I, _I, _I, _P]
-        c.velox_grouped_glu.argtypes = [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _F, _F, _P]
+        c.velox_grouped_glu.argtypes = [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _F, _F, _I, _P]
         c.velox_grouped_down.argtypes = [_P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]
         c.velox_routed_combine.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _I, _P, _P, _I, _P]
-        c.velox_routed_products_bf16.argtypes = [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _F, _F, _P]
+        c.velox_routed_products_bf16.argtypes = [_P, _P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _F, _F, _I, _P]
         c.velox_routed_combine_norm.argtypes = [_P, _P, _P, _I, _I, _I, _I, _I, _P, _P, _I, _P, _P, _F, _F, _P, _P]
         c.velox_routed_combine_norm.restype = _I
         c.velox_add_sinusoid.argtypes = [_P, _P, _P, _I, _I, _P]
@@ -165,11 +165,17 @@ class HipOps:
         c.velox_embed_copies.argtypes = [_P, _P, _I, _P, _I, _I, _I, _F, _I, _P]
         c.velox_gated_act_mul.argtypes = [_P, _P, _I, _I, _I, _I, _P]
         c.velox_short_conv.argtypes = [_P, _I, _I, _P, _I, _P, _P, _P, _P, _I, _I, _I, _I, _I, _P]
-        c.velox_rotate_pad_write.argtypes = [_P, _I, _P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P]
+        c.velox_rotate_pad_write.argtypes = [_P, _I, _P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P]
         c.velox_recurrence_prepare.argtypes = [_P, _I, _I, _I, _I, _I, _I, _I, _F, _P, _I, _I, _I, _I, _I, _P, _P, _F, _P, _I, _I, _I, _P, _P, _P, _I, _P]
         c.velox_linear_scan.argtypes = [_P, _P, _I, _I, _I, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P]
         c.velox_linear_scan_lanes.argtypes = [_I]
         c.velox_gated_head_norm.argtypes = [_P, _P, _F, _P, _I, _I, _I, _I, _P, _I, _I, _I, _I, _P]
+        c.velox_embed_bigram.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _P, _P, _P, _P, _P]
+        c.velox_add_dynamic_tanh.argtypes = [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, ctypes.c_longlong, _P, _I, _P]
+        c.velox_scale.argtypes = [_P, ctypes.c_longlong, _F, _P]
+        c.velox_activation.argtypes = [_P, _P, ctypes.c_longlong, _I, _I, _P]
+        for fn in (c.velox_embed_bigram, c.velox_add_dynamic_tanh, c.velox_scale, c.velox_activation):
+            fn.restype = _I
         for fn in (c.velox_stream_norm, c.velox_embed_copies, c.velox_gated_act_mul, c.velox_short_conv, c.velox_rotate_pad_write, c.velox_recurrence_prepare,
                    c.velox_linear_scan, c.velox_linear_scan_lanes, c.velox_gated_head_norm):
             fn.restype = _I
@@ -188,7 +194,7 @@ class HipOps:
         lib = self._attention.get(key)
         if lib is None:
             lib = ctypes.CDLL(build.ensure_attention(head_dim, biased=bool(biased)))
-            lib.velox_paged_attention.argtypes = [_P, _I, _P, _P, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _I, _P, _I, _P]
+            lib.velox_paged_attention.argtypes = [_P, _I, _P, _P, _P, _I, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _I, _P, _I, _P, _P]
             lib.velox_attention_biased.restype = _I
             lib.velox_paged_attention.restype = _I
             lib.velox_attention_head_dim.restype = _I
@@ -361,6 +367,89 @@ class HipOps:
             raise KernelError(f"place_tokens: {count} pairs do not fit dest [{dest.numel()}] and source [{source.numel()}]")
         status = self._core.velox_place_tokens(_ptr(ids), _ptr(dest), _ptr(source), _ptr(tokens), int(count), ids.numel(), tokens.numel(), self._stream())
         self._launched(status, "place_tokens")
+
+    def embed_bigram(self, token_ids, table, bigram, scale, buckets, mul_prev, mul_cur, positions, cu_q, slots, state, max_q_len) -> torch.Tensor:
+        """``table[ids[t]] * scale + bigram[row(t)]`` in float32, ``row(t) = (previous * mul_prev + ids[t] * mul_cur) mod buckets`` and
+        ``buckets`` at position 0; the token before a portion's first one is ``state[slots[b], 0]`` (int32 ``[slots, 1]``), which is
+        then set to the portion's last token."""
+        self._check("token_ids", token_ids, torch.int32)
+        self._check("table", table)
+        if token_ids.dim() != 1 or table.dim() != 2:
+            raise KernelError("embed_bigram: token_ids must be [T] and the table [V, H]")
+        tokens = token_ids.shape[0]
+        vocab, hidden = table.shape
+        self._check("bigram", bigram, table.dtype, (int(buckets) + 1, hidden))
+        self._check("positions", positions, torch.int32, (tokens,))
+        self._check("cu_q", cu_q, torch.int32)
+        num_seqs = cu_q.shape[0] - 1
+        self._check("slots", slots, torch.int32, (num_seqs,))
+        self._check("state", state, torch.int32)
+        if state.dim() != 2 or state.shape[1] != 1:
+            raise KernelError(f"embed_bigram: the state holds one token per slot, [slots, 1]; got {tuple(state.shape)}")
+        if not 1 <= max_q_len <= tokens or num_seqs < 1:
+            raise KernelError(f"embed_bigram: max_q_len={max_q_len} outside [1, {tokens}]")
+        out = torch.empty((tokens, hidden), dtype=torch.float32, device=self.device)
+        status = self._core.velox_embed_bigram(_ptr(token_ids), _ptr(table), _ptr(bigram), _ptr(out), tokens, num_seqs, int(max_q_len), hidden, vocab,
+                                               _code(table.dtype), float(scale), int(buckets), int(mul_prev), int(mul_cur), _ptr(positions), _ptr(cu_q),
+                                               _ptr(slots), _ptr(state), self._stream())
+        self._launched(status, "embed_bigram")
+        return out
+
+    def add_dynamic_tanh(self, residual, delta, weight, bias, alpha, out_dtype, rows=None):
+        """``residual += delta`` (float32, in place; with ``rows`` nothing is changed and only those rows are worked), then
+        ``tanh(alpha x) * weight + bias``; ``alpha`` is a float32 tensor of one number on the device.  ``delta`` as for ``add_rmsnorm``."""
+        self._check("residual", residual, torch.float32)
+        if residual.dim() != 2:
+            raise KernelError("add_dynamic_tanh: residual must be [T, H]")
+        tokens, hidden = residual.shape
+        self._check("weight", weight, torch.float32, (hidden,))
+        self._check("bias", bias, torch.float32, (hidden,))
+        self._check("alpha", alpha, torch.float32)
+        if alpha.numel() != 1:
+            raise KernelError("add_dynamic_tanh: alpha is one number")
+        partials, partial_stride = 1, 0
+        second = None
+        if isinstance(delta, SumOf):
+            delta, second = delta.first, delta.second
+            self._check("second term of the delta", second, None, (tokens, hidden))
+        if delta is not None:
+            if delta.dim() == 3:
+                partials, partial_stride = delta.shape[0], tokens * hidden
+                self._check("delta", delta, torch.float32, (partials, tokens, hidden), align=16)
+            else:
+                self._check("delta", delta, None, (tokens, hidden))
+        count = tokens
+        if rows is not None:
+            self._check("rows", rows, torch.int32)
+            count = rows.shape[0]
+        out = torch.empty((count, hidden), dtype=out_dtype, device=self.device)
+        delta_code = _code(delta.dtype) if delta is not None else _code(out_dtype)
+        status = self._core.velox_add_dynamic_tanh(_ptr(residual), _ptr(delta), _ptr(rows), _ptr(weight), _ptr(bias), _ptr(alpha), _ptr(out), count, hidden,
+                                                   delta_code, _code(out_dtype), partials, partial_stride, _ptr(second),
+                                                   _code(second.dtype) if second is not None else 0, self._stream())
+        self._launched(status, "add_dynamic_tanh")
+        return out
+
+    def scale_(self, x: torch.Tensor, factor: float) -> torch.Tensor:
+        """``x *= factor`` in place, float32."""
+        self._check("x", x, torch.float32)
+        self._launched(self._core.velox_scale(_ptr(x), x.numel(), float(factor), self._stream()), "scale")
+        return x
+
+    _ACTIVATION_CODES = {"relu2": 1}
+
+    def activation(self, x: torch.Tensor, kind: str) -> torch.Tensor:
+        """The activation of a unit without a gate branch, float32 arithmetic with one rounding: ``relu2`` = ``relu(x)^2``."""
+        if kind not in self._ACTIVATION_CODES:
+            raise KernelError(f"activation {kind!r} is not implemented")
+        self._check("x", x)
+        out = torch.empty_like(x)
+        self._launched(self._core.velox_activation(_ptr(x), _ptr(out), x.numel(), self._ACTIVATION_CODES[kind], _code(x.dtype), self._stream()), "activation")
+        return out
+
+    def linear_act(self, x, weight, out_dtype: torch.dtype, kind: str) -> torch.Tensor:
+        """``act(x @ weight^T)``: the product, then the activation's kernel."""
+        return self.activation(self.linear(x, weight, None, out_dtype), kind)
 
     def _norm(self, residual, delta, rows, weight, eps, out_dtype):
         self._check("residual", residual, torch.float32)
@@ -862,9 +951,10 @@ class HipOps:
         self._launched(status, "short_conv")
         return out
 
-    def rotate_pad_write(self, qkv, num_heads, num_kv_heads, dim, vdim, cached_dim, positions, cos, sin, slot_mapping, k_cache, v_cache, block_size, write_kv=True):
+    def rotate_pad_write(self, qkv, num_heads, num_kv_heads, dim, vdim, cached_dim, positions, cos, sin, slot_mapping, k_cache, v_cache, block_size, write_kv=True,
+                         interleaved=False):
         """Rotates the first ``2 * cos.shape[1]`` channels of every q and k head of ``qkv`` [T, heads * dim + kv_heads * (dim + vdim)]
-        (channel i with i + half), writes k and v into the pages at ``cached_dim`` channels a head (zeros in the padding)
+        (channel i with i + half, or 2i with 2i + 1 when ``interleaved``), writes k and v into the pages at ``cached_dim`` channels a head (zeros in the padding)
         and returns q as [T, heads * cached_dim]."""
         self._check("qkv", qkv)
         tokens = qkv.shape[0]
@@ -891,7 +981,7 @@ class HipOps:
         q = torch.empty((tokens, num_heads * cached_dim), dtype=qkv.dtype, device=self.device)
         status = self._core.velox_rotate_pad_write(_ptr(qkv), width, _ptr(q), _ptr(positions), _ptr(cos), _ptr(sin), half, _ptr(slot_mapping) if write_kv else _P(0),
                                                    _ptr(k_cache) if write_kv else _P(0), _ptr(v_cache) if write_kv else _P(0), tokens, num_heads, num_kv_heads,
-                                                   dim, vdim, cached_dim, int(block_size), int(bool(write_kv)), _code(qkv.dtype), self._stream())
+                                                   dim, vdim, cached_dim, int(block_size), int(bool(write_kv)), _code(qkv.dtype), int(bool(interleaved)), self._stream())
         self._launched(status, "rotate_pad_write")
         return q
 
@@ -1090,12 +1180,14 @@ class HipOps:
 
     # -- attention over a cached latent -----------------------------------------------------------
     def latent_rotate_write(self, projected, num_heads, dim, rot_dim, kv_rank, cached_dim, down_offset, positions, cos, sin, interleaved,
-                            norm_weight, eps, slot_mapping, k_cache, v_cache, block_size) -> torch.Tensor:
+                            norm_weight, eps, slot_mapping, k_cache, v_cache, block_size, q_latent=None):
         """Rows of ``projected`` hold ``num_heads`` queries of ``dim`` plain and ``rot_dim`` rotated channels and, at
         ``down_offset`` (-1: none, nothing is written to the cache), a latent of ``kv_rank`` and a shared key part of
         ``rot_dim`` channels.  Returns the queries the attention kernels read, ``[T, num_heads * cached_dim]``: of every head
         the channels from ``kv_rank`` on are written here (the rotated part, then zeros), the first ``kv_rank`` are left
-        for ``head_linear``.  The normed latent and the rotated shared part go into the cache."""
+        for ``head_linear``.  The normed latent and the rotated shared part go into the cache.  ``num_heads`` = 0: no
+        queries.  ``q_latent = (offset, rank, weight)``: those columns of every row are RMS-normed with the weight as well;
+        then ``(queries, normed [T, rank])`` comes back."""
         if projected.dim() != 2:
             raise KernelError("latent_rotate_write: rows are [T, width]")
         tokens, width = projected.shape
@@ -1106,7 +1198,7 @@ class HipOps:
             self._check("cos", cos, torch.float32)
             self._check("sin", sin, torch.float32, tuple(cos.shape))
             half = cos.shape[1]
-        if (num_heads * (dim + rot_dim) > width or 2 * half > rot_dim or cached_dim < kv_rank + rot_dim
+        if (num_heads < 0 or num_heads * (dim + rot_dim) > width or 2 * half > rot_dim or cached_dim < kv_rank + rot_dim
                 or (down_offset >= 0 and down_offset + kv_rank + rot_dim > width)):
             raise KernelError(f"latent_rotate_write: rows of {width} do not hold {num_heads} x ({dim} + {rot_dim}) queries and a latent of {kv_rank} + {rot_dim} at {down_offset}")
         if down_offset >= 0:
@@ -1115,17 +1207,35 @@ class HipOps:
             pages = k_cache.shape[0]
             self._check("k_cache", k_cache, projected.dtype, (pages, 1, block_size, cached_dim))
             self._check("v_cache", v_cache, projected.dtype, (pages, 1, cached_dim, block_size))
+        normed, norm2 = None, (0, 0, None)
+        if q_latent is not None:
+            norm2 = (int(q_latent[0]), int(q_latent[1]), q_latent[2])
+            self._check("q_latent weight", norm2[2], torch.float32, (norm2[1],))
+            if norm2[0] < 0 or norm2[1] < 1 or norm2[0] + norm2[1] > width:
+                raise KernelError(f"latent_rotate_write: columns {norm2[0]} .. {norm2[0] + norm2[1]} lie outside rows of {width}")
+            normed = torch.empty((tokens, norm2[1]), dtype=projected.dtype, device=self.device)
         queries = torch.empty((tokens, num_heads * cached_dim), dtype=projected.dtype, device=self.device)
         status = self._core.velox_latent_rotate_write(
             _ptr(projected), width, _ptr(queries), tokens, num_heads, dim, rot_dim, kv_rank, cached_dim, int(down_offset), _ptr(positions), _ptr(cos), _ptr(sin),
             half, int(bool(interleaved)), _ptr(norm_weight) if down_offset >= 0 else _P(0), float(eps), _ptr(slot_mapping) if down_offset >= 0 else _P(0),
-            _ptr(k_cache) if down_offset >= 0 else _P(0), _ptr(v_cache) if down_offset >= 0 else _P(0), int(block_size), _code(projected.dtype), self._stream())
+            _ptr(k_cache) if down_offset >= 0 else _P(0), _ptr(v_cache) if down_offset >= 0 else _P(0), int(block_size), _code(projected.dtype),
+            norm2[0], norm2[1], _ptr(norm2[2]), _ptr(normed), self._stream())
         self._launched(status, "latent_rotate_write")
-        return queries
+        return queries if q_latent is None else (queries, normed)
 
-    def head_linear(self, x, x_head_stride, x_offset, maps, out, out_head_stride, out_offset, gate=None, gate_offset=0) -> torch.Tensor:
+    def latent_write(self, projected, rot_dim, kv_rank, cached_dim, down_offset, positions, cos, sin, interleaved, norm_weight, eps, slot_mapping,
+                     k_cache, v_cache, block_size, q_latent=None):
+        """The cache write of ``latent_rotate_write`` without any queries (the same kernel): norm of the latent at
+        ``down_offset``, rotation of the shared key part, both into the pages.  ``q_latent = (offset, rank, weight)``: those
+        columns come back RMS-normed with the weight, ``[T, rank]`` (the queries' own latent, on its way to its second product)."""
+        result = self.latent_rotate_write(projected, 0, 0, rot_dim, kv_rank, cached_dim, down_offset, positions, cos, sin, interleaved, norm_weight, eps,
+                                          slot_mapping, k_cache, v_cache, block_size, q_latent=q_latent)
+        return None if q_latent is None else result[1]
+
+    def head_linear(self, x, x_head_stride, x_offset, maps, out, out_head_stride, out_offset, gate=None, gate_offset=0, gate_per_head=False) -> torch.Tensor:
         """``out[t, g * out_head_stride + out_offset + j] = sum_k x[t, g * x_head_stride + x_offset + k] * maps[g, j, k]``, times
-        ``sigmoid(gate[t, gate_offset + g * n + j])`` when ``gate`` is given: one small product per head, the heads at fixed
+        ``sigmoid(gate[t, gate_offset + g * n + j])`` when ``gate`` is given (``gate_per_head``: ``sigmoid(gate[t, gate_offset + g])``,
+        one number for all outputs of a head): one small product per head, the heads at fixed
         strides inside the rows of ``x`` and ``out`` (written in place, other columns untouched)."""
         if x.dim() != 2 or out.dim() != 2 or maps.dim() != 3 or x.shape[0] != out.shape[0]:
             raise KernelError("head_linear: x and out are [T, width], maps is [groups, n, k]")
@@ -1140,19 +1250,26 @@ class HipOps:
         if gate is not None:
             self._check("gate", gate, x.dtype)
             gate_width = gate.shape[1]
-            if gate.dim() != 2 or gate.shape[0] != x.shape[0] or gate_offset < 0 or gate_offset + groups * n > gate_width:
+            if gate.dim() != 2 or gate.shape[0] != x.shape[0] or gate_offset < 0 or gate_offset + (groups if gate_per_head else groups * n) > gate_width:
                 raise KernelError("head_linear: the gate's columns lie outside its rows")
         status = self._core.velox_head_linear(_ptr(x), x.shape[1], int(x_head_stride), int(x_offset), _ptr(maps), _ptr(out), out.shape[1], int(out_head_stride),
-                                              int(out_offset), _ptr(gate), gate_width, int(gate_offset), x.shape[0], groups, n, k, _code(x.dtype), self._stream())
+                                              int(out_offset), _ptr(gate), gate_width, int(gate_offset), x.shape[0], groups, n, k, _code(x.dtype), int(bool(gate_per_head)), self._stream())
         self._launched(status, "head_linear")
         return out
 
     # -- routed experts ---------------------------------------------------------------------------
-    def route_top(self, logits: torch.Tensor, top: int, score: str = "sigmoid", renormalize: bool = False, correction: Optional[torch.Tensor] = None):
+    def route_top(self, logits: torch.Tensor, top: int, score: str = "sigmoid", renormalize: bool = False, correction: Optional[torch.Tensor] = None,
+                  groups: Optional[Tuple[int, int]] = None, norm_floor: float = 0.0):
         """float32 ``logits`` [T, E] -> (int32 choices [T, top], float32 weights [T, top]): the ``top`` largest scores
         (``sigmoid`` or ``softmax`` over all experts), ties to the lower index, divided by their sum when ``renormalize``.
-        ``correction`` (float32 [E]) is added to the scores for the choice only: the weights are the scores without it."""
+        ``correction`` (float32 [E]) is added to the scores for the choice only: the weights are the scores without it.
+        ``groups = (count, keep)``: the experts form ``count`` equal groups of neighbours (64 at most), a group's score is the sum of
+        its two largest choice scores, and only experts of the ``keep`` best groups can be chosen.  ``norm_floor`` is added to
+        the sum that renormalised weights are divided by."""
         self._check("logits", logits, torch.float32)
+        count, keep = (int(groups[0]), int(groups[1])) if groups else (0, 0)
+        if groups and (not 1 <= count <= 64 or logits.shape[-1] % count or not 1 <= keep <= count or keep * (logits.shape[-1] // count) < top):
+            raise KernelError(f"route_top: groups={groups} do not fit {logits.shape[-1]} experts and top={top}")
         if correction is not None:
             self._check("correction", correction, torch.float32, (logits.shape[-1],))
         if logits.dim() != 2 or not 1 <= top <= logits.shape[1] or score not in ("sigmoid", "softmax"):
@@ -1161,7 +1278,7 @@ class HipOps:
         choice = torch.empty((tokens, top), dtype=torch.int32, device=self.device)
         weight = torch.empty((tokens, top), dtype=torch.float32, device=self.device)
         self._launched(self._core.velox_route_top(_ptr(logits), _ptr(choice), _ptr(weight), tokens, experts, int(top), int(score == "softmax"),
-                                                  int(bool(renormalize)), _ptr(correction), self._stream()), "route_top")
+                                                  int(bool(renormalize)), _ptr(correction), count, keep, float(norm_floor), self._stream()), "route_top")
         return choice, weight
 
     def routed_plan_elems(self, max_num_tokens: int, top: int, experts: int) -> int:
@@ -1169,7 +1286,7 @@ class HipOps:
         return int(self._core.velox_routed_plan_elems(int(max_num_tokens) * int(top), int(experts)))
 
     def routed_experts(self, x, choice, weight, gate_up_weight, down_weight, num_experts: int, scale_input: bool, shared, out_dtype, workspace=None,
-                       unit: Tuple[float, float, float] = (1.0, float("inf"), 0.0), identity_experts: int = 0, output_norm=None):
+                       unit: Tuple[float, float, float] = (1.0, float("inf"), 0.0), identity_experts: int = 0, output_norm=None, ungated: Optional[str] = None):
         """``sum_k unit_{choice[t, k]}(weight[t, k] x[t])`` (or the weight on the unit's output), plus ``shared``: the pairs
         are sorted by expert on the device, two grouped products run every expert on its rows, and each token's results
         are added in the order of its choices.  ``gate_up_weight`` [E * 2F, H] (per expert gate rows, then up rows),
@@ -1177,18 +1294,23 @@ class HipOps:
         shift)`` with ``g = min(gate, limit)``, ``u = clamp(up, -limit, limit)``.  ``identity_experts``: choices from
         ``num_experts`` on are experts without tensors whose result is ``weight[t, k] x[t]``; the plan leaves them out and
         the last kernel adds them in their turn.  ``output_norm`` (an ``OutputNormSink``): the last kernel norms the sum in
-        float32 and adds it to the sink's residual; what comes back is then a ``ResidualCopy`` of the updated residual."""
+        float32 and adds it to the sink's residual; what comes back is then a ``ResidualCopy`` of the updated residual.
+        ``ungated`` (``"relu2"``): the units have no gate branch, ``W_down act(W_up x)``; ``gate_up_weight`` is then [E * F, H]."""
         alpha, limit, shift = (float(v) for v in unit)
+        if ungated is not None and ungated not in self._ACTIVATION_CODES:
+            raise KernelError(f"routed_experts: activation {ungated!r} is not implemented")
+        act_code = self._ACTIVATION_CODES[ungated] if ungated is not None else 0
+        branches = 1 if ungated is not None else 2
         if not limit > 0 or identity_experts < 0:
             raise KernelError(f"routed_experts: unit={unit}, identity_experts={identity_experts}")
         tokens, hidden = x.shape
         top = choice.shape[1]
         pairs = tokens * top
-        inter = gate_up_weight.shape[0] // (2 * num_experts)
+        inter = gate_up_weight.shape[0] // (branches * num_experts)
         self._check("x", x)
         self._check("choice", choice, torch.int32, (tokens, top))
         self._check("weight", weight, torch.float32, (tokens, top))
-        self._check("gate_up_weight", gate_up_weight, x.dtype, (num_experts * 2 * inter, hidden))
+        self._check("gate_up_weight", gate_up_weight, x.dtype, (num_experts * branches * inter, hidden))
         self._check("down_weight", down_weight, x.dtype, (num_experts * hidden, inter))
         if shared is not None:
             self._check("shared", shared, out_dtype, (tokens, hidden))
@@ -1201,7 +1323,7 @@ class HipOps:
             plan = torch.empty(elems, dtype=torch.int32, device=self.device)
         on_matrix_cores = x.dtype == torch.bfloat16 and hidden % 8 == 0 and inter % 8 == 0 and self.use_grouped_mfma
         # tiles of 128 rows for the matrix cores when the experts have that many rows on average (W is then read half as often)
-        tile_rows = 128 if on_matrix_cores and pairs >= 128 * num_experts and 2 * inter > 128 and hidden > 128 else 64
+        tile_rows = 128 if on_matrix_cores and pairs >= 128 * num_experts and branches * inter > 128 and hidden > 128 else 64
         # few pairs: the plan's kernel also copies the rows into its order, and the step runs one kernel less
         ordered = torch.empty((pairs, hidden), dtype=x.dtype, device=self.device) if on_matrix_cores else None
         copied_by_plan = on_matrix_cores and pairs <= self.FEW_PAIRS
@@ -1214,12 +1336,12 @@ class HipOps:
             # bfloat16 rows of whole 16-byte pieces: sorted copies of the rows, then both products on the matrix cores
             self._launched(self._core.velox_routed_products_bf16(_P(0) if copied_by_plan else _ptr(x), _ptr(gate_up_weight), _ptr(down_weight), _ptr(ordered), _ptr(act), _ptr(y), _ptr(plan),
                                                                  _ptr(weight), pairs, num_experts, top, inter, hidden, int(bool(scale_input)), tile_rows,
-                                                                 alpha, limit, shift, self._stream()), "routed_products")
+                                                                 alpha, limit, shift, act_code, self._stream()), "routed_products")
             # (a weight on the output is applied by the last kernel: the second product is the same kernel either way)
             return self._routed_combine(y, plan, shared, tokens, top, num_experts, hidden, out_dtype, x if identity_experts else None, weight,
                                         scale_rows=not scale_input, output_norm=output_norm)
         self._launched(self._core.velox_grouped_glu(_ptr(x), _ptr(gate_up_weight), _ptr(act), _ptr(plan), _ptr(weight), pairs, num_experts, top, inter, hidden,
-                                                    int(bool(scale_input)), _code(x.dtype), alpha, limit, shift, self._stream()), "grouped_glu")
+                                                    int(bool(scale_input)), _code(x.dtype), alpha, limit, shift, act_code, self._stream()), "grouped_glu")
         self._launched(self._core.velox_grouped_down(_ptr(act), _ptr(down_weight), _ptr(y), _ptr(plan), _ptr(weight), pairs, num_experts, top, hidden, inter,
                                                      int(not scale_input), _code(x.dtype), self._stream()), "grouped_down")
         return self._routed_combine(y, plan, shared, tokens, top, num_experts, hidden, out_dtype, x if identity_experts else None, weight,
@@ -1293,15 +1415,19 @@ class HipOps:
 
     def paged_attention(self, qkv, num_heads, num_kv_heads, head_dim, k_cache, v_cache, block_size, block_tables, cu_q, kv_lens,
                         max_q_len, max_kv_len, scale, window, all_decode, workspace, splits: Optional[int] = None, decode_prefix: int = 0,
-                        portions_max_kv_len: Optional[int] = None, distance_bias: Optional[torch.Tensor] = None):
+                        portions_max_kv_len: Optional[int] = None, distance_bias: Optional[torch.Tensor] = None, sinks: Optional[torch.Tensor] = None):
         """Attention of every token of the step over its sequence's keys in the cache.  ``decode_prefix``: how many of the
         first sequences bring exactly one token (the engine puts decoded tokens before portions of prompts).  In a mixed
         step those run through the streaming kernel with their keys split over workgroups, the others through the
         general kernel: a single token behind many keys would otherwise be one workgroup's long walk that the
         whole step waits for.  ``portions_max_kv_len``: the most keys any sequence behind that prefix holds (default: ``max_kv_len``).
         ``distance_bias``: float32 ``[num_heads, L]``, added to the scaled scores: a key ``n`` positions behind the query reads
-        column ``min(n, L - 1)`` of its query head's row (the kernels' build for it is loaded by ``attention_library(d, True)``)."""
+        column ``min(n, L - 1)`` of its query head's row (the kernels' build for it is loaded by ``attention_library(d, True)``).
+        ``sinks``: float32 ``[num_heads]``; ``exp(sinks[h])`` joins the denominator of every softmax of head ``h`` (a sink has no key
+        and no value and is not scaled)."""
         tokens = qkv.shape[0]
+        if sinks is not None:
+            self._check("sinks", sinks, torch.float32, (num_heads,))
         width = qkv.shape[1] if qkv.dim() == 2 else -1  # rows may carry keys and values after the queries
         if width not in (num_heads * head_dim, (num_heads + 2 * num_kv_heads) * head_dim):
             raise KernelError(f"paged_attention: rows of {width} elements hold neither the queries nor queries, keys and values")
@@ -1341,7 +1467,7 @@ class HipOps:
             status = self._core.velox_plain_attention(_ptr(qkv), width, _ptr(k_cache), _ptr(v_cache), _ptr(block_tables), block_tables.shape[1], _ptr(cu_q),
                                                       _ptr(kv_lens), _ptr(out), num_seqs, tokens, num_heads, num_kv_heads, head_dim,
                                                       block_size.bit_length() - 1, float(scale), int(window or 0), _code(qkv.dtype), _ptr(distance_bias), bias_len,
-                                                      self._stream())
+                                                      _ptr(sinks), self._stream())
             self._launched(status, "plain_attention")
             return out
         lib = self.attention_library(head_dim, distance_bias is not None)
@@ -1371,7 +1497,7 @@ class HipOps:
                 _ptr(cu_q[first_seq:]), _ptr(kv_lens[first_seq:]), _ptr(rows_out), _ptr(part_o), _ptr(part_lse), count,
                 num_tokens if decode_only else tokens, longest, int(max_kv_len), num_heads, num_kv_heads,
                 block_size.bit_length() - 1, float(scale), int(window or 0), splits, 0 if decode_only else first_token, _code(qkv.dtype),
-                _ptr(distance_bias), bias_len, self._stream())
+                _ptr(distance_bias), bias_len, _ptr(sinks), self._stream())
             self._launched(status, "paged_attention")
 
         if not all_decode and splits is None and 0 < decode_prefix < num_seqs and group <= 16:
