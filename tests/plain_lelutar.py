@@ -39,7 +39,7 @@ def rms_unit(x: torch.Tensor, eps: float) -> torch.Tensor:
 
 def embed(config: dict, w: Dict[str, torch.Tensor], tokens: List[int]) -> torch.Tensor:
     """x_t = E[token_t] * scale + B[(prev * mul_prev + token * mul_cur) mod buckets]; the first token reads the last row."""
-    spec = config["embedding"]
+    spec = config.get("embedding") or {}
     ids = torch.tensor(tokens, dtype=torch.long)
     x = w["embed"][ids] * float(spec.get("scale", 1.0))
     bigram = spec.get("bigram")
