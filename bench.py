@@ -16,6 +16,9 @@ over the steps in which all of them decode, ``..._frac``: that step's share of t
 ``e2e_b<B>_p512_g256``: generated tokens / wall time with the prompts' time included, which is how
 the reference's ``benchmark.py:204`` counts).
 
+``--design lelutar`` measures the Lelutar design (norms without statistics, a hashed table of token pairs beside the embedding, grouped-query
+attention with two head sizes beside attention over a latent with a sink and a gate per head, ungated experts chosen among the best groups)
+beside Tiverax with the same experts and the dense decoder with the same heads.
 ``--design gosulorn`` measures the Gosulorn design (residual streams, attention over a sliding window beside a gated delta rule, gated
 linear attention, delta rules; every mixer's memory a state of fixed size or a window's pages) beside the dense decoder of the same width,
 depth, heads and feed-forward size; ``--design dipisun`` does for the Dipisun design what ``--design tiverax`` does for Tiverax, beside Tiverax with the same experts and
@@ -301,6 +304,34 @@ def gosulorn_config(size: dict) -> dict:
     return {"architecture": "Gosulorn", "vocab": DESIGN_VOCAB, "width": size["width"], "norm": {"eps": 1e-5}, "streams": size["streams"], "layers": layers}
 
 
+# Layer sizes for --design lelutar: eight layers, twice (attention with a dense feed-forward, attention, attention over a latent without
+# positions, the same with a rotated key part, these three with experts in groups); the last two layers run the weights of the
+# two before them again.  Beside it: Tiverax with the same experts in every layer, and the dense decoder with the same heads.
+LELUTAR_SIZES = {
+    "2k": dict(width=2048, heads=16, kv_heads=4, dim=128, vdim=128, latent_dim=64, rot_dim=32, latent_vdim=64, kv_rank=128, q_rank=512, ff=5632,
+               experts=16, top=2, groups=(4, 2), expert_ff=1408, buckets=65521),
+    "4k": dict(width=4096, heads=32, kv_heads=8, dim=128, vdim=128, latent_dim=96, rot_dim=32, latent_vdim=128, kv_rank=224, q_rank=768, ff=11008,
+               experts=32, top=4, groups=(8, 4), expert_ff=1408, buckets=65521),
+}
+
+
+def lelutar_config(size: dict) -> dict:
+    stretch = {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}
+    attention = {"heads": size["heads"], "kv_heads": size["kv_heads"], "dim": size["dim"], "vdim": size["vdim"], "scale": size["dim"] ** -0.5,
+                 "rot": {"dims": size["dim"], "base": 1e6, "scaling": stretch}}
+    latent = {"heads": size["heads"], "dim": size["latent_dim"], "vdim": size["latent_vdim"], "kv_rank": size["kv_rank"], "q_rank": size["q_rank"],
+              "scale": size["latent_dim"] ** -0.5}
+    latent_2 = dict(latent, rot_dim=size["rot_dim"], scale=(size["latent_dim"] + size["rot_dim"]) ** -0.5, rot={"dims": size["rot_dim"], "base": 1e6, "scaling": stretch})
+    dense = {"kind": "dense", "ff": size["ff"]}
+    routed = {"kind": "moe", "router": {"experts": size["experts"], "top": size["top"], "groups": {"count": size["groups"][0], "keep": size["groups"][1]}},
+              "expert": {"ff": size["expert_ff"]}}
+    order = (("attention", attention, dense), ("attention", attention, routed), ("latent_attention", latent, routed), ("latent_attention_2", latent_2, routed))
+    layers = [{"type": kind, "mixer": mixer, "mlp": mlp} for kind, mixer, mlp in order * 2]
+    layers[6]["weights_of"], layers[7]["weights_of"] = 2, 3
+    return {"architecture": "Lelutar", "vocab": DESIGN_VOCAB, "width": size["width"], "norm": {"eps": 1e-5}, "logit_scale": 0.5,
+            "embedding": {"scale": size["width"] ** 0.5, "bigram": {"buckets": size["buckets"], "mul_prev": 1000003, "mul_cur": 998244353 % 65536}}, "layers": layers}
+
+
 def tiverax_all_routed(size: dict) -> dict:
     """Tiverax at the width of ``size`` with the same experts per layer and per token (no shared expert, no dense layers)."""
     config = tiverax_config(dict(TIVERAX_SIZES["2k" if size["width"] == 2048 else "4k"], experts=size["experts"], top=size["top"], expert_ff=size["expert_ff"]))
@@ -317,6 +348,10 @@ def designs_at(design: str, name: str):
     if design == "gosulorn":
         size = GOSULORN_SIZES[name]
         return (("gosulorn", gosulorn_config(size)), ("qwen2", qwen2_like(dict(size, rot_dim=0))))
+    if design == "lelutar":
+        size = LELUTAR_SIZES[name]
+        dense = dict(width=size["width"], heads=size["heads"], kv_heads=size["kv_heads"], dim=size["dim"], rot_dim=0, ff=size["top"] * size["expert_ff"])
+        return (("lelutar", lelutar_config(size)), ("tiverax", tiverax_all_routed(size)), ("qwen2", qwen2_like(dense)))
     size = DIPISUN_SIZES[name]
     dense = dict(width=size["width"], heads=size["heads"], kv_heads=size["kv_heads"], dim=size["dim"], rot_dim=0, ff=size["top"] * size["expert_ff"])
     return (("dipisun", dipisun_config(size)), ("tiverax", tiverax_all_routed(size)), ("qwen2", qwen2_like(dense)))
@@ -366,7 +401,7 @@ def main() -> int:
     parser.add_argument("--shape", default="7b", choices=sorted(SHAPES), help="layer sizes: the headline is 7b; 1.5b and 32b are the reference's other two")
     parser.add_argument("--far", action="store_true",
                         help="further sizes under `points`: decode at batch 1 and 8 behind 32,256 tokens, a prefill of 8,192 tokens, and a decode step of a true float32 run (batch 8)")
-    parser.add_argument("--design", default=None, choices=["tiverax", "dipisun", "gosulorn"],
+    parser.add_argument("--design", default=None, choices=["tiverax", "dipisun", "gosulorn", "lelutar"],
                         help="instead of the headline: prefill and decode of this design at real layer sizes beside the framework's closest models of equal size")
     parser.add_argument("--only", default="", help="with --design: which of the models that are measured side by side (names with commas between them; default: all)")
     parser.add_argument("--sizes", default="2k,4k", help="with --design: which of the sizes (2k, 4k = the models' widths)")
@@ -380,7 +415,7 @@ def main() -> int:
         points = design_points(args)
         first = args.sizes.split(",")[0]
         head = points.get(f"{args.design}_{first}") or next(iter(points.values()))
-        sizes = {"tiverax": TIVERAX_SIZES, "dipisun": DIPISUN_SIZES, "gosulorn": GOSULORN_SIZES}[args.design]
+        sizes = {"tiverax": TIVERAX_SIZES, "dipisun": DIPISUN_SIZES, "gosulorn": GOSULORN_SIZES, "lelutar": LELUTAR_SIZES}[args.design]
         print(json.dumps({
             "metric": "decode_tokens_per_second", "value": head["decode_tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": args.steps,
             "warmup": args.warmup, "ms_per_step": head["decode_ms"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,

@@ -49,6 +49,7 @@ __global__ void __launch_bounds__(256) route_top_kernel(const float* __restrict_
     for (int e = lane; e < experts; e += 64) sum += expf(z[e] - shift);
     denom = wave_sum(sum);
   }
+  const int used = (experts + 63) >> 6;  // registers of `score` that hold experts at all: the loops below stop there
   float score[ROUTE_PER_LANE];
 #pragma unroll
   for (int u = 0; u < ROUTE_PER_LANE; ++u) {
@@ -63,11 +64,25 @@ __global__ void __launch_bounds__(256) route_top_kernel(const float* __restrict_
     // lane g ends up with group g's score (group_count <= 64); every group's two largest by two rounds over the wave
     const int per = experts / group_count;
     float mine = -INFINITY;  // (lanes beyond the groups never win)
+    if (used == 1 && (per & (per - 1)) == 0) {
+      // one expert per lane and groups that are aligned runs of a power of two of lanes: all groups at once, the two
+      // largest of a run by exchanges inside the run
+      float first = score[0], second = -INFINITY;
+      for (int offset = 1; offset < per; offset <<= 1) {
+        const float of = __shfl_xor(first, offset, 64), os = __shfl_xor(second, offset, 64);
+        second = fmaxf(fminf(first, of), fmaxf(second, os));
+        first = fmaxf(first, of);
+      }
+      const float sum = per > 1 ? first + second : first;
+      const float of_group = __shfl(sum, (lane * per) & 63, 64);
+      if (lane < group_count) mine = of_group;
+    } else
     for (int gidx = 0; gidx < group_count; ++gidx) {
       const int lo = gidx * per, hi = lo + per;
       float first = -INFINITY, second = -INFINITY;  // this lane's two largest inside the group
 #pragma unroll
       for (int u = 0; u < ROUTE_PER_LANE; ++u) {
+        if (u >= used) break;
         const int e = lane + 64 * u;
         if (e >= lo && e < hi) {
           const float v = score[u];
@@ -106,6 +121,7 @@ __global__ void __launch_bounds__(256) route_top_kernel(const float* __restrict_
     }
 #pragma unroll
     for (int u = 0; u < ROUTE_PER_LANE; ++u) {
+      if (u >= used) break;
       const int e = lane + 64 * u;
       if (e < experts && !((allowed >> (e / per)) & 1ull)) score[u] = -INFINITY;
     }
@@ -115,8 +131,10 @@ __global__ void __launch_bounds__(256) route_top_kernel(const float* __restrict_
     float best = -INFINITY;
     int best_e = 0x7fffffff;
 #pragma unroll
-    for (int u = 0; u < ROUTE_PER_LANE; ++u)
+    for (int u = 0; u < ROUTE_PER_LANE; ++u) {
+      if (u >= used) break;
       if (score[u] > best) { best = score[u]; best_e = lane + 64 * u; }  // (ascending e within a lane: the first of equals stays)
+    }
 #pragma unroll
     for (int offset = 32; offset > 0; offset >>= 1) {
       const float other = __shfl_xor(best, offset, 64);
@@ -124,8 +142,10 @@ __global__ void __launch_bounds__(256) route_top_kernel(const float* __restrict_
       if (other > best || (other == best && other_e < best_e)) { best = other; best_e = other_e; }
     }
 #pragma unroll
-    for (int u = 0; u < ROUTE_PER_LANE; ++u)
+    for (int u = 0; u < ROUTE_PER_LANE; ++u) {
+      if (u >= used) break;
       if (lane + 64 * u == best_e) score[u] = -INFINITY;
+    }
     // (the weight is the score without the correction: the same expression as above, so the same value)
     if (best_e >= experts) best_e = 0;  // (only when every score left is a NaN: stay inside the row)
     if (correction) best = softmax ? expf(z[best_e] - shift) / denom : 1.f / (1.f + expf(-z[best_e]));

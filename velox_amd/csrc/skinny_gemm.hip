@@ -183,6 +183,7 @@ struct RowScale {
   int blocks;
   float inv_width, eps;
   int act = 0;  // the gate's activation where a kernel stores act(gate) * up: 0 SiLU, 1 the tanh form of GELU
+  int ungated = 0;  // the plain product's epilogue: ungated_act(sum + bias, ungated), 0 = none (see common.h)
 };
 
 // How a workgroup adds a row's sums: wave v takes the blocks [v * share, (v + 1) * share), lane (g, row) of it every fourth
@@ -306,6 +307,7 @@ __global__ void __launch_bounds__(WAVES * 64) skinny_gemm_kernel(const bf16_t* _
       if (row_n + j >= n) break;
       float v = sum[j];
       if (bias) v += bias[row_n + j];
+      if constexpr (!GLU) v = ungated_act(v, rs.ungated);  // (a unit without a gate branch: the activation on the float32 sum)
       out[(size_t)col_m * n + row_n + j] = from_f32<TO>(v);
       four[j] = from_f32<bf16_t>(v);
     }
@@ -369,11 +371,13 @@ static int launch_skinny(const void* a, const void* w, const float* bias, void* 
 // a_packed != 0: a is in the lanes' order (see packed_row_offset); only with M <= 16.
 extern "C" int velox_skinny_gemm_bf16(const void* a, const void* w, const float* bias, void* out, int m, int n, int k, int out_dtype,
                                       int waves, int row_tiles, int packed, const float* scale_partial, int scale_blocks,
-                                      float inv_width, float eps, int a_packed, hipStream_t stream) {
+                                      float inv_width, float eps, int a_packed, int ungated, hipStream_t stream) {
+  // ungated: the activation of a unit without a gate branch as the epilogue (VELOX_ACT_RELU2), 0 = none
   if (m <= 0 || n <= 0) return 0;
   if (k % 64 != 0 || m > 64 || (scale_partial != nullptr && (m > 16 || scale_blocks > ROW_SCALE_BLOCKS)) || (a_packed && m > 16)) return -1;
   if (scale_partial != nullptr && waves < 8) waves = 8;  // (rows are scaled by the eight-wave kernels)
-  const RowScale rs{scale_partial, scale_blocks, inv_width, eps};
+  RowScale rs{scale_partial, scale_blocks, inv_width, eps};
+  rs.ungated = ungated;
 #define PICK(RT, CT, W) return launch_skinny<RT, CT, W>(a, w, bias, out, m, n, k, out_dtype, packed != 0, rs, a_packed, stream)
   if (m <= 16 && row_tiles >= 4) {
     if (waves >= 8) PICK(4, 1, 8);

@@ -115,7 +115,7 @@ class HipOps:
         c.velox_rope_kv_write_partial_bf16.argtypes = [_P, _P, _I, _P, _P, _P, _P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P]
         c.velox_rope_kv_write_partial_bf16.restype = _I
         c.velox_gemm_fma.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P]
-        c.velox_skinny_gemm_bf16.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P, _I, _F, _F, _I, _P]
+        c.velox_skinny_gemm_bf16.argtypes = [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P, _I, _F, _F, _I, _I, _P]
         c.velox_skinny_residual_norm_bf16.argtypes = [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _P, _P]
         c.velox_skinny_residual_norm_bf16.restype = _I
         c.velox_row_scale_apply.argtypes = [_P, _P, _I, _F, _F, _P, _I, _I, _P]
@@ -448,7 +448,20 @@ class HipOps:
         return out
 
     def linear_act(self, x, weight, out_dtype: torch.dtype, kind: str) -> torch.Tensor:
-        """``act(x @ weight^T)``: the product, then the activation's kernel."""
+        """``act(x @ weight^T)`` for a unit without a gate branch: for decode-sized bfloat16 batches one kernel (the activation
+        on the float32 sums is the product's epilogue, so the sums are rounded once), else the product and the
+        activation's kernel."""
+        if kind not in self._ACTIVATION_CODES:
+            raise KernelError(f"activation {kind!r} is not implemented")
+        plain, prepared = _weight_of(weight)
+        x = self.materialize(x)
+        skinny_rows = 16 if plain.shape[0] > 8192 else 32  # (as ``linear`` sends its products)
+        if (self.use_skinny_gemm and x.dim() == 2 and x.dtype == torch.bfloat16 and plain.dtype == torch.bfloat16 and out_dtype == torch.bfloat16
+                and x.shape[0] <= skinny_rows and x.shape[1] % 64 == 0 and x.shape[1] == plain.shape[1]):
+            self._check("x", x, align=16)
+            self._check("weight", plain, align=16)
+            return self.skinny_gemm(x, plain, None, out_dtype, packed=prepared.copy(1) if prepared is not None else None,
+                                    x_packed=self._packed_rows_of(x, x.shape[1]), ungated=kind)
         return self.activation(self.linear(x, weight, None, out_dtype), kind)
 
     def _norm(self, residual, delta, rows, weight, eps, out_dtype):
@@ -728,10 +741,11 @@ class HipOps:
         return padded.view(matrices, tiles, 16, k // 64, 4, 2, 8).permute(0, 1, 3, 5, 4, 2, 6).contiguous().view(-1)
 
     def skinny_gemm(self, x, weight, bias, out_dtype, waves: Optional[int] = None, row_tiles: Optional[int] = None, packed: Optional[torch.Tensor] = None, n: Optional[int] = None,
-                    row_scale: Optional[DeferredNorm] = None, x_packed: Optional[torch.Tensor] = None):
+                    row_scale: Optional[DeferredNorm] = None, x_packed: Optional[torch.Tensor] = None, ungated: Optional[str] = None):
         """Few rows (M <= 64) times a bfloat16 weight: the weight-streaming kernel of the decode step.  ``packed`` is
         ``pack_rows(weight)``, used instead of ``weight`` when given (``n`` = rows of the weight).  ``row_scale``: ``x`` is
-        its ``.x`` and the result rows are scaled as it says (M <= 16)."""
+        its ``.x`` and the result rows are scaled as it says (M <= 16).  ``ungated``: the activation of a unit without a gate
+        branch (``relu2``) on the float32 sums, as the product's epilogue."""
         m, k = x.shape
         n = weight.shape[0] if weight is not None else n
         if packed is not None:
@@ -759,7 +773,7 @@ class HipOps:
             raise KernelError("skinny_gemm: the packed activations do not match M and K")
         status = self._core.velox_skinny_gemm_bf16(_ptr(x if x_packed is None else x_packed), _ptr(weight_arg), _ptr(bias), _ptr(out), m, n, k, _code(out_dtype),
                                                    int(waves), int(row_tiles), 1 if packed is not None else 0, *self._scale_args(row_scale),
-                                                   int(x_packed is not None), self._stream())
+                                                   int(x_packed is not None), self._ACTIVATION_CODES[ungated] if ungated else 0, self._stream())
         self._launched(status, "skinny_gemm")
         return out
 
