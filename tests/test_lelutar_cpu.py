@@ -36,12 +36,18 @@ def test_configuration_is_read_layer_by_layer_and_refused_where_it_cannot_run():
     assert type(model.blocks[2].feed_forward).__name__ == "NoFeedForward" and model.blocks[1].feed_forward.groups == (3, 2)
     assert model.blocks[1].mixer.rot_dim == 0 and model.blocks[2].mixer.rot_dim == 8 and model.blocks[1].mixer.gate_per_head
     assert model.head.scale == 1.5 and model.embedding.scale == 1.75
+    # a layer may name a layer that itself runs another's weights, or one that comes later: the owner is found either way
+    chained = copy.deepcopy(CONFIGS["A"])
+    chained["layers"][5]["weights_of"] = 3
+    chained["layers"][2], chained["layers"][4] = chained["layers"][4], chained["layers"][2]
+    chained["layers"][2]["weights_of"] = 4
+    assert [e.layer for e in build_model(config_from_dict(chained), torch.float32, "cpu", max_position=64).schedule] == [0, 1, 2, 0, 2, 0]
     plain_embedding = build_model(config_from_dict(CONFIGS["B"]), torch.float32, "cpu", max_position=32)
     assert type(plain_embedding.embedding).__name__ == "TableEmbedding" and len(plain_embedding.cache_needs()) == 4 and plain_embedding.head.scale == 1.0
     for change, message in (
         (lambda c: c["layers"][3].update(weights_of=1), "type"),
         (lambda c: c["layers"][3].update(weights_of=3), "weights_of"),
-        (lambda c: c["layers"][5].update(weights_of=3), "weights_of"),
+        (lambda c: (c["layers"][0].update(weights_of=3), c["layers"][3].update(weights_of=0)), "weights_of"),
         (lambda c: c["layers"][0].update(type="other"), "type"),
         (lambda c: c["layers"][0]["mlp"].update(kind="other"), "kind"),
         (lambda c: c["layers"][1]["mlp"]["router"].update(top=9), "top"),

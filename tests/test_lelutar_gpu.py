@@ -42,7 +42,7 @@ def close(got, want, dtype, scale=1.0):
 # kernels alone
 # ----------------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("buckets,mul_prev,mul_cur,width", [(31, 7, 3, 72), (1, 5, 5, 6), (257, 2000000011, 1999999973, 321)])
+@pytest.mark.parametrize("buckets,mul_prev,mul_cur,width", [(31, 7, 3, 72), (1, 5, 5, 6), (257, 2000000011, 1999999973, 321), (65521, (1 << 40) + 3, (1 << 33) + 5, 8)])
 def test_pair_table_embedding_with_its_state(ops, dtype, buckets, mul_prev, mul_cur, width):
     """Steps of portions and single tokens of three sequences: rows and the state after every step equal the reference's."""
     ref, dt = TorchOps(), DTYPES[dtype]

@@ -554,7 +554,8 @@ extern "C" int velox_row_scale_apply(const void* x, const float* sums, int block
 // embedding with a hashed table of token pairs:
 //   out[t, :] = float(table[ids[t], :]) * scale + float(bigram[row(t), :])
 //   row(t) = buckets                                                  at position 0
-//          = (previous * mul_prev + ids[t] * mul_cur) mod buckets     otherwise (64-bit arithmetic)
+//          = (previous * mul_prev + ids[t] * mul_cur) mod buckets     otherwise; the caller hands the multipliers reduced mod
+//            buckets (0 <= mul < buckets < 2^31), the ids are reduced here, so the 64-bit sum of the two products cannot overflow
 // `previous` is ids[t - 1] inside a sequence's portion and, for a portion's first token, what the sequence's state
 // holds (state[slots[b]]); the workgroup that works a portion's first token reads the state and THEN sets it to the
 // portion's last token, so no other workgroup touches the entry.  Grid: (row blocks of a sequence, sequences); an id
@@ -584,7 +585,9 @@ __global__ void __launch_bounds__(256) embed_bigram_kernel(const int* __restrict
     for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = __builtin_nanf("");
     return;
   }
-  const long long row = positions[t] == 0 ? buckets : ((long long)previous * mul_prev + (long long)id * mul_cur) % buckets;
+  long long before = (long long)previous % buckets;
+  if (before < 0) before += buckets;  // (an id outside the table in the row before: any row, never out of bounds)
+  const long long row = positions[t] == 0 ? buckets : (before * mul_prev + ((long long)id % buckets) * mul_cur) % buckets;
   const T* src = table + (size_t)id * hidden;
   const T* pair = bigram + (size_t)row * hidden;
   for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = to_f32(src[i]) * scale + to_f32(pair[i]);
@@ -594,7 +597,7 @@ extern "C" int velox_embed_bigram(const int* ids, const void* table, const void*
                                   int vocab, int table_dtype, float scale, int buckets, int mul_prev, int mul_cur, const int* positions, const int* cu_q,
                                   const int* slots, int* state, hipStream_t stream) {
   if (tokens <= 0 || num_seqs <= 0) return 0;
-  if (buckets < 1 || mul_prev < 0 || mul_cur < 0 || max_q_len < 1 || num_seqs > 65535) return -1;
+  if (buckets < 1 || mul_prev < 0 || mul_cur < 0 || mul_prev >= buckets || mul_cur >= buckets || max_q_len < 1 || num_seqs > 65535) return -1;
   dim3 grid(max_q_len, num_seqs);
   if (table_dtype == VELOX_BF16)
     embed_bigram_kernel<bf16_t><<<grid, 256, 0, stream>>>(ids, (const bf16_t*)table, (const bf16_t*)bigram, out, hidden, vocab, scale, buckets, mul_prev,

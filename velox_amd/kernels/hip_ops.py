@@ -388,9 +388,12 @@ class HipOps:
             raise KernelError(f"embed_bigram: the state holds one token per slot, [slots, 1]; got {tuple(state.shape)}")
         if not 1 <= max_q_len <= tokens or num_seqs < 1:
             raise KernelError(f"embed_bigram: max_q_len={max_q_len} outside [1, {tokens}]")
+        if not 1 <= int(buckets) < 2 ** 31:
+            raise KernelError(f"embed_bigram: buckets={buckets} must lie between 1 and 2^31 - 1")
         out = torch.empty((tokens, hidden), dtype=torch.float32, device=self.device)
+        # (the multipliers reduced mod buckets, exactly, whatever their size or sign: the kernel's 64-bit sum then cannot overflow)
         status = self._core.velox_embed_bigram(_ptr(token_ids), _ptr(table), _ptr(bigram), _ptr(out), tokens, num_seqs, int(max_q_len), hidden, vocab,
-                                               _code(table.dtype), float(scale), int(buckets), int(mul_prev), int(mul_cur), _ptr(positions), _ptr(cu_q),
+                                               _code(table.dtype), float(scale), int(buckets), int(mul_prev) % int(buckets), int(mul_cur) % int(buckets), _ptr(positions), _ptr(cu_q),
                                                _ptr(slots), _ptr(state), self._stream())
         self._launched(status, "embed_bigram")
         return out

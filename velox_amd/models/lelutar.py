@@ -114,24 +114,30 @@ class LelutarConfig(ModelConfig):
         bigram = None
         if embedding.get("bigram") is not None:
             bigram = tuple(require(embedding["bigram"], key, int) for key in ("buckets", "mul_prev", "mul_cur"))
-            if bigram[0] < 1 or min(bigram[1:]) < 0:
-                raise ConfigError("embedding.bigram: buckets must be positive, the multipliers not negative")
+            if not 1 <= bigram[0] < 2 ** 31:
+                raise ConfigError("embedding.bigram: buckets must be positive (and below 2^31)")
         listed = raw.get("layers")
         if not isinstance(listed, list) or not listed:
             raise ConfigError("config.json: 'layers' must list at least one layer")
-        layers: List[Dict[str, Any]] = []
+        layers: List[Optional[Dict[str, Any]]] = [None] * len(listed)
+        # whose tensors a layer runs: itself, or the layer its ``weights_of`` names (followed to a layer that owns tensors)
+        owners: List[int] = []
+        for index, entry in enumerate(listed):
+            if not isinstance(entry, dict) or entry.get("type") not in _TYPES:
+                raise ConfigError(f"layers[{index}].type={entry.get('type') if isinstance(entry, dict) else entry!r} is not a layer of this design ({', '.join(_TYPES)})")
+            owner, seen = index, set()
+            while listed[owner].get("weights_of") is not None:
+                seen.add(owner)
+                owner = int(listed[owner]["weights_of"])
+                if not 0 <= owner < len(listed) or owner in seen or not isinstance(listed[owner], dict):
+                    raise ConfigError(f"layers[{index}].weights_of must lead to a layer that owns its tensors")
+            if listed[owner].get("type") != entry["type"]:
+                raise ConfigError(f"layers[{index}].a layer that runs layer {owner}'s weights is of its type")
+            owners.append(owner)
         for index, entry in enumerate(listed):
             where = f"layers[{index}]."
-            kind = entry.get("type")
-            if kind not in _TYPES:
-                raise ConfigError(f"{where}type={kind!r} is not a layer of this design ({', '.join(_TYPES)})")
-            if entry.get("weights_of") is not None:
-                owner = int(entry["weights_of"])
-                if not 0 <= owner < index or layers[owner]["owner"] != owner:
-                    raise ConfigError(f"{where}weights_of must name an earlier layer that owns its tensors")
-                if layers[owner]["type"] != kind:
-                    raise ConfigError(f"{where}a layer that runs layer {owner}'s weights is of its type")
-                layers.append(dict(layers[owner], owner=owner))
+            kind = entry["type"]
+            if owners[index] != index:
                 continue
             mixer = _section(entry, "mixer", where)
             keys = ("heads", "kv_heads", "dim", "vdim") if kind == "attention" else ("heads", "dim", "vdim", "kv_rank", "q_rank")
@@ -151,7 +157,10 @@ class LelutarConfig(ModelConfig):
                       "mlp": _feed_forward(entry.get("mlp"), where)}
             if not parsed["scale"] > 0:
                 raise ConfigError(f"{where}mixer.scale must be positive")
-            layers.append(parsed)
+            layers[index] = parsed
+        for index, owner in enumerate(owners):
+            if owner != index:
+                layers[index] = dict(layers[owner], owner=owner)
         return LelutarConfig(architecture=architecture_name(raw), raw=dict(raw), width=width, vocab=vocab, norm_eps=eps, embedding_scale=scale,
                              bigram=bigram, logit_scale=float(raw.get("logit_scale", 1.0)), layers=layers)
 
@@ -167,11 +176,12 @@ def lelutar_spec(config: LelutarConfig, max_position: Optional[int] = None) -> M
     key_of: Dict[tuple, str] = {}
     layers: List[LayerSpec] = []
     schedule: List[ScheduleEntry] = []
-    place: Dict[int, int] = {}  # configuration index of a weight-owning layer -> its place in ``layers``
+    owning = [index for index, layer in enumerate(config.layers) if layer["owner"] == index]
+    place: Dict[int, int] = {index: at for at, index in enumerate(owning)}  # configuration index of a weight-owning layer -> its place in ``layers``
     for index, layer in enumerate(config.layers):
-        if layer["owner"] != index:
-            schedule.append(ScheduleEntry(place[layer["owner"]]))
-            continue
+        schedule.append(ScheduleEntry(place[layer["owner"]]))
+    for index in owning:
+        layer = config.layers[index]
         position = None
         if layer["rotation"] is not None:
             if layer["rotation"] not in key_of:  # layers with the same rotation share its tables
@@ -197,10 +207,8 @@ def lelutar_spec(config: LelutarConfig, max_position: Optional[int] = None) -> M
             feed_forward = PartSpec.of("routed_experts", hidden_size=width, intermediate_size=mlp["ff"], num_experts=mlp["experts"], top=mlp["top"],
                                        score="sigmoid", renormalize=True, renormalize_floor=RENORMALIZE_FLOOR, scale_input=False, ungated="relu2",
                                        groups=mlp["groups"], expert_names=("e{e}.up", "e{e}.down"), router_name="router", correction_name="correction")
-        place[index] = len(layers)
         layers.append(LayerSpec(prefix=f"l{index}.", mixer=mixer, feed_forward=feed_forward, mixer_norm=norm, ff_norm=norm, position=position,
                                 arrangement="pre_norm", mixer_prefix="mix.", feed_forward_prefix="mlp.", mixer_norm_prefix="norm1", ff_norm_prefix="norm2"))
-        schedule.append(ScheduleEntry(place[index]))
     if config.bigram is not None:
         embedding = PartSpec.of("bigram_table", scale=config.embedding_scale, buckets=config.bigram[0], mul_prev=config.bigram[1], mul_cur=config.bigram[2],
                                 bigram_name="bigram")
