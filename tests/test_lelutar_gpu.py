@@ -225,7 +225,7 @@ def _paged_case(nh, nkv, d, q_lens, kv_lens, page, dt, seed=0):
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("nh,nkv,d,q_lens,kv_lens", [
     (5, 1, 80, [1, 1, 1], [70, 1, 300]),                 # single tokens, one workgroup per sequence
-    (7, 1, 112, [1, 1], [5000, 2300]),                   # single tokens behind keys that are split over workgroups and merged
+    (7, 1, 96, [1, 1], [5000, 2300]),                    # single tokens behind keys that are split over workgroups and merged
     (4, 2, 64, [9, 30, 2], [9, 155, 40]),                # short portions: the staged kernel
     (8, 2, 64, [600, 500], [600, 1500]),                 # long portions of 64 channels (bfloat16: tiles loaded straight into LDS)
     (16, 1, 128, [300], [4500]),                         # a portion behind keys that are split
