@@ -9,7 +9,7 @@ import torch
 
 import plain_lelutar as plain
 import replay_cases as rc
-from lelutar_cases import CONFIGS, PAGE_SIZE, attention, dense, latent, latent_2, moe, prompts, random_weights, rot, tensor_shapes, write_folder
+from lelutar_cases import CONFIGS, PAGE_SIZE, prompts, random_weights, tensor_shapes, write_folder
 from torch_ops import TorchOps
 from velox_amd import Engine, EngineConfig, Request, SamplingParams
 from velox_amd.config.model_config import ConfigError
