@@ -248,25 +248,26 @@ def test_a_mechanism_left_out_would_show(tmp_path):
     assert changed(lambda c: c["layers"][3].pop("weights_of"), lambda w: w.update({k.replace("l0.", "l3."): v + 0.05 for k, v in list(w.items()) if k.startswith("l0.")})) > 0.05
 
 
-def test_a_key_far_back_is_found_from_a_portion_and_from_a_single_token(tmp_path):
-    """One early token is made to stand out for one head of every kind of mixer (its key is loud along one direction, and
-    late queries point along it), hundreds of tokens and many pages back: the logits 260 tokens on depend on it, and the
-    framework finds it from a portion and from single tokens alike."""
+@pytest.mark.parametrize("far_at,length", [(3, 300), (0, 90), (4, 90), (7, 90), (8, 90), (16, 90)])
+def test_a_key_far_back_is_found_from_a_portion_and_from_a_single_token(tmp_path, far_at, length):
+    """One early token is made to stand out (its embedding is loud, so its keys are), hundreds of tokens and many pages
+    back, or at a page's first or last place (pages of 4 tokens): the late logits depend on it, and the framework finds
+    it from a portion and from single tokens alike, written by one step and read by later ones."""
     config = copy.deepcopy(CONFIGS["A"])
     weights = random_weights(config, 9)
-    tokens = prompts(config["vocab"], [300], seed=5)["r0"]
-    tokens[3] = 96
-    tokens = [t if t != 96 or i == 3 else 95 for i, t in enumerate(tokens)]  # token 96 occurs once, at position 3
+    tokens = [t if t != 96 else 95 for t in prompts(config["vocab"], [length], seed=5)["r0"]]
+    tokens[far_at] = 96  # token 96 occurs once
     weights["embed"][96] *= 4.0
     right = plain.forward(config, weights, tokens)
     other = list(tokens)
-    other[3] = 5
+    other[far_at] = 5
     moved = (right[-40:] - plain.forward(config, weights, other)[-40:]).abs().amax(-1)
     assert float(moved.min()) > 0.02  # (every late position feels the early token)
     folder = write_folder(tmp_path / "far", config, seed=9, weights=weights)
     requests = {"r0": tokens}
-    for trace in (rc.whole(requests), rc.tail_one_by_one(requests, tail=45), rc.changing_portions(requests, sizes=(64, 2, 100, 3, 50, 1, 2, 38, 1))):
-        replayer = Replayer(folder, "float32", 304, block_size=4, device="cpu", ops=TorchOps(), max_live=2)
+    cuts = (64, 2, 100, 3, 50, 1, 2, 38, 1) if length == 300 else (far_at + 1, 2, 30, 1, 3, 17, 2)
+    for trace in (rc.whole(requests), rc.tail_one_by_one(requests, tail=45), rc.changing_portions(requests, sizes=cuts)):
+        replayer = Replayer(folder, "float32", length + 4, block_size=4, device="cpu", ops=TorchOps(), max_live=2)
         got = rc.collect(trace, rc.run_trace(replayer, trace), requests)
         torch.testing.assert_close(got["r0"], right, **TOL)
 

@@ -287,28 +287,29 @@ def test_all_ways_of_cutting_on_the_gpu(tmp_path, name, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-def test_a_key_far_back_behind_split_keys(tmp_path, dtype):
+@pytest.mark.parametrize("far_at,length", [(3, 1100), (0, 200), (15, 200), (16, 200), (17, 200), (64, 200)])
+def test_a_key_far_back_behind_split_keys_or_at_a_page_border(tmp_path, dtype, far_at, length):
     """One early token is made loud; 1,100 tokens on, where single tokens read their keys in splits that a kernel merges
-    (sinks included), the logits still depend on it and equal the plain model's, from a portion and from single tokens."""
+    (sinks included), or from a page's first or last place (pages of 16 tokens), the logits still depend on it and equal
+    the plain model's, from a portion and from single tokens, written by one step and read by later ones."""
     config = CONFIGS["C"]
     weights = random_weights(config, 9)
-    tokens = prompts(config["vocab"], [1100], seed=5)["r0"]
-    tokens = [t if t != 159 else 158 for t in tokens]
-    tokens[3] = 159
+    tokens = [t if t != 159 else 158 for t in prompts(config["vocab"], [length], seed=5)["r0"]]
+    tokens[far_at] = 159
     weights["embed"][159] *= 4.0
     folder = write_folder(tmp_path / "far", config, seed=9, dtype=dtype, weights=weights)
     config, weights = plain.read_folder(folder)
     right = plain.forward(config, weights, tokens)
     other = list(tokens)
-    other[3] = 5
+    other[far_at] = 5
     moved = (right[-30:] - plain.forward(config, weights, other)[-30:]).abs().amax(-1)
     assert float(moved.median()) > 0.05
     requests = {"r0": tokens}
-    for label, trace in (("whole", rc.whole(requests)), ("tail", rc.tail_one_by_one(requests, tail=40)),
-                         ("portions", rc.changing_portions(requests, sizes=(500, 2, 300, 3, 250, 1, 2, 38, 1, 1, 1, 1)))):
-        replayer = Replayer(folder, dtype, 1104, block_size=16, max_live=2)
+    cuts = (500, 2, 300, 3, 250, 1, 2, 38, 1, 1, 1, 1) if length > 1000 else (far_at + 1, 2, 100, 1, 3, 33, 2)
+    for label, trace in (("whole", rc.whole(requests)), ("tail", rc.tail_one_by_one(requests, tail=40)), ("portions", rc.changing_portions(requests, sizes=cuts))):
+        replayer = Replayer(folder, dtype, length + 16, block_size=16, max_live=2)
         got = rc.collect(trace, rc.run_trace(replayer, trace), requests)
-        rows_close(got["r0"][-200:], right[-200:], dtype, f"far {label}")
+        rows_close(got["r0"][-150:], right[-150:], dtype, f"far {label}")
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
